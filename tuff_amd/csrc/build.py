@@ -39,6 +39,7 @@ MODULES = {
     "recurrent": "recurrent.hip",
     "moe": "moe.hip",
     "hyper": "hyper.hip",
+    "postnorm": "postnorm.hip",
     "latent": "latent.hip",
     "sampling": "sampling.hip",
 }

@@ -258,14 +258,16 @@ TUFF_EXPORT int tuff_glu(const void* gu, int in_dt, void* act, int dt, int n_tok
     return launch_status();
 }
 
-// out[t, c] = f(in[t, c]) * (row_gate ? g(row_gate[t * gate_stride]) : 1): an activation, optionally times one
-// number a row (g: gate_kind, or -1 for the number as it is).  in and out may be the same memory.
+// out[t, c] = f(in[t, c] + (col_bias ? col_bias[c] : 0)) * (row_gate ? g(row_gate[t * gate_stride]) : 1): an activation
+// (after a bias per column, where given), optionally times one number a row (g: gate_kind, or -1 for the number as
+// it is).  in and out may be the same memory.
 template <typename TI, typename TO>
 __global__ void act_rows_kernel(const TI* __restrict__ in, TO* __restrict__ out, long long n, int N, int kind,
-                                const float* __restrict__ row_gate, int gate_stride, int gate_kind) {
+                                const float* __restrict__ row_gate, int gate_stride, int gate_kind,
+                                const float* __restrict__ col_bias) {
     const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= n) return;
-    float v = activation(to_f32(in[i]), kind);
+    float v = activation(to_f32(in[i]) + (col_bias ? col_bias[i % N] : 0.f), kind);
     if (row_gate) {
         const float g = row_gate[(i / N) * gate_stride];
         v *= gate_kind < 0 ? g : activation(g, gate_kind);
@@ -274,11 +276,11 @@ __global__ void act_rows_kernel(const TI* __restrict__ in, TO* __restrict__ out,
 }
 
 TUFF_EXPORT int tuff_act_rows(const void* in, int in_dt, void* out, int out_dt, long long rows, int N, int kind,
-                              const float* row_gate, int gate_stride, int gate_kind, hipStream_t stream) {
+                              const float* row_gate, int gate_stride, int gate_kind, const float* col_bias, hipStream_t stream) {
     const long long n = rows * N;
     if (n <= 0) return 0;
     dim3 grid((unsigned)ceil_div_ll(n, 256)), block(256);
-#define LAUNCH(TI, TO) hipLaunchKernelGGL((act_rows_kernel<TI, TO>), grid, block, 0, stream, (const TI*)in, (TO*)out, n, N, kind, row_gate, gate_stride, gate_kind)
+#define LAUNCH(TI, TO) hipLaunchKernelGGL((act_rows_kernel<TI, TO>), grid, block, 0, stream, (const TI*)in, (TO*)out, n, N, kind, row_gate, gate_stride, gate_kind, col_bias)
     if (in_dt == DT_F32 && out_dt == DT_F32) LAUNCH(float, float);
     else if (in_dt == DT_F32) LAUNCH(float, bf16_t);
     else if (out_dt == DT_F32) LAUNCH(bf16_t, float);

@@ -37,7 +37,7 @@ _SIGNATURES = {
         "tuff_scatter_i32": [_c_void_p, _c_int, _c_void_p, _c_int, _c_void_p, _c_int, _c_void_p],
         "tuff_dyt": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_void_p, _c_int, _c_int, _c_void_p],
         "tuff_glu": [_c_void_p, _c_int, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_void_p, _c_float, _c_float, _c_void_p],
-        "tuff_act_rows": [_c_void_p, _c_int, _c_void_p, _c_int, _c_ll, _c_int, _c_int, _c_void_p, _c_int, _c_int, _c_void_p],
+        "tuff_act_rows": [_c_void_p, _c_int, _c_void_p, _c_int, _c_ll, _c_int, _c_int, _c_void_p, _c_int, _c_int, _c_void_p, _c_void_p],
         "tuff_pad_cols": [_c_void_p, _c_void_p, _c_int, _c_ll, _c_int, _c_int, _c_void_p],
     },
     "recurrent": {
@@ -53,6 +53,8 @@ _SIGNATURES = {
                             _c_int, _c_int, _c_int, _c_ll, _c_ll, _c_void_p],
         "tuff_head_norm_gate": [_c_void_p, _c_void_p, _c_int, _c_void_p, _c_int, _c_int, _c_int, _c_void_p, _c_int, _c_int, _c_int,
                                 _c_float, _c_void_p],
+        "tuff_forget_scan": [_c_void_p, _c_int, _c_ll, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p,
+                             _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p],
     },
     "moe": {
         "tuff_moe_route": [_c_void_p, _c_int, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_void_p],
@@ -97,7 +99,14 @@ _SIGNATURES = {
     "attention": {
         "tuff_attention_general": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_void_p, _c_int,
                                    _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
-                                   _c_float, _c_void_p, _c_void_p, _c_int, _c_void_p],
+                                   _c_float, _c_void_p, _c_void_p, _c_int, _c_void_p, _c_void_p, _c_int, _c_void_p],
+        "tuff_head_mix_gate": [_c_void_p, _c_int, _c_void_p, _c_void_p, _c_int, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int,
+                               _c_void_p],
+    },
+    "postnorm": {
+        "tuff_post_norm_add": [_c_void_p, _c_void_p, _c_void_p, _c_float, _c_float, _c_void_p, _c_void_p, _c_float, _c_void_p,
+                               _c_int, _c_int, _c_int, _c_int, _c_void_p],
+        "tuff_normed_mean2": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_float, _c_float, _c_void_p, _c_int, _c_int, _c_void_p],
     },
     "hyper": {
         "tuff_hc_step": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_void_p,
@@ -396,9 +405,10 @@ def glu(gu: torch.Tensor, act: torch.Tensor, activation: str, bias: Optional[tor
 
 
 def act_rows(inp: torch.Tensor, out: torch.Tensor, activation: str, row_gate: Optional[torch.Tensor] = None,
-             gate_col: int = 0, gate_activation: Optional[str] = None) -> None:
-    """out = activation(inp), each row times gate_activation(row_gate[row, gate_col]) where row_gate
-    (float32 [rows, *]) is given (gate_activation None: the number as it is).  inp may be out."""
+             gate_col: int = 0, gate_activation: Optional[str] = None, bias: Optional[torch.Tensor] = None) -> None:
+    """out = activation(inp [+ bias]), each row times gate_activation(row_gate[row, gate_col]) where row_gate
+    (float32 [rows, *]) is given (gate_activation None: the number as it is).  bias: float32 [N], a number a column,
+    added before the activation.  inp may be out."""
     rows, N = out.shape
     _gpu("inp", inp, shape=(rows, N))
     _gpu("out", out)
@@ -410,7 +420,7 @@ def act_rows(inp: torch.Tensor, out: torch.Tensor, activation: str, row_gate: Op
         gp, stride = row_gate.data_ptr() + 4 * gate_col, row_gate.shape[1]
     _check(load("elementwise").tuff_act_rows(
         inp.data_ptr(), _dt(inp), out.data_ptr(), _dt(out), rows, N, ACTIVATIONS[activation], gp, stride,
-        -1 if gate_activation is None else ACTIVATIONS[gate_activation], _stream()), "act_rows")
+        -1 if gate_activation is None else ACTIVATIONS[gate_activation], _opt("bias", bias, torch.float32, (N,)), _stream()), "act_rows")
 
 
 def pad_cols(inp: torch.Tensor, width: int) -> torch.Tensor:
@@ -793,15 +803,29 @@ def kv_write(k, v, k_cache, v_cache, slot_mapping, *, Hkv, hd, page_size, vd=Non
 
 # -------------------------------------------------------------------------- attention
 def attention_general(q, k_cache, v_cache, out, *, block_table, req_of_token, positions,
-                      H, Hkv, hd, page_size, window=0, scale=None, vd=None, sinks=None, slopes=None) -> None:
+                      H, Hkv, hd, page_size, window=0, scale=None, vd=None, sinks=None, slopes=None,
+                      log_distance=None, all_values: bool = False) -> None:
     """vd: width of a value where it is not the keys'.  sinks: float32 [H], a logit per head that counts
     once in the softmax's denominator and has no value.  slopes: float32 [H]; slopes[h] * (position - key) is
-    taken off head h's scaled scores.  v_cache None: the values are the first vd channels of the key rows."""
+    taken off head h's scaled scores.  v_cache None: the values are the first vd channels of the key rows.
+    log_distance: (r1, r2), float32 [H] each; r1[h] * ln(1 + r2[h] * (position - key)) is taken off head h's scaled
+    scores.  all_values: every query head's weights are applied to the values of every kv head; out is then float32
+    [T, H * Hkv * vd] (head, kv head, channel), for head_mix_gate."""
     T = q.shape[0]
     dt = q.dtype
     vd = hd if vd is None else int(vd)
     _gpu("q", q, shape=(T, H * hd))
-    _gpu("out", out, dt, (T, H * vd))
+    if all_values:
+        if v_cache is None:
+            raise KernelError("attention: all_values needs a value cache")
+        _gpu("out", out, torch.float32, (T, H * Hkv * vd))
+    else:
+        _gpu("out", out, dt, (T, H * vd))
+    r1 = r2 = None
+    if log_distance is not None:
+        r1, r2 = log_distance
+        _gpu("log_distance r1", r1, torch.float32, (H,))
+        _gpu("log_distance r2", r2, torch.float32, (H,))
     P = k_cache.shape[0]
     _gpu("k_cache", k_cache, dt, (P, Hkv, page_size, hd))
     if v_cache is None:
@@ -824,7 +848,66 @@ def attention_general(q, k_cache, v_cache, out, *, block_table, req_of_token, po
         q.data_ptr(), k_cache.data_ptr(), None if v_cache is None else v_cache.data_ptr(), out.data_ptr(), _dt(q),
         block_table.data_ptr(), block_table.shape[1], req_of_token.data_ptr(), positions.data_ptr(),
         T, H, Hkv, hd, vd, page_size, int(window or 0), float(scale), None if sinks is None else sinks.data_ptr(),
-        None if slopes is None else slopes.data_ptr(), int(v_cache is None), _stream()), "attention_general")
+        None if slopes is None else slopes.data_ptr(), int(v_cache is None),
+        None if r1 is None else r1.data_ptr(), None if r2 is None else r2.data_ptr(), int(all_values), _stream()), "attention_general")
+
+
+def head_mix_gate(o, out, *, H, Hkv, vd, talk=None, gates=None) -> None:
+    """After attention: out[t, h] = sigmoid(gates[t, h]) * o[t, h] (o [T, H * vd]), or, with talk float32 [H, H] and
+    o float32 [T, H * Hkv * vd] as attention_general(all_values=True) leaves it,
+    out[t, h] = sigmoid(gates[t, h]) * sum_g talk[h, g] o[t, g, kv head of h].  gates float32 [T, >= H] (rows of one
+    stride; the first H columns count) or None for no gate; out [T, H * vd] of the compute type."""
+    T = out.shape[0]
+    _gpu("out", out, shape=(T, H * vd))
+    if talk is not None:
+        _gpu("talk", talk, torch.float32, (H, H))
+        _gpu("o", o, torch.float32, (T, H * Hkv * vd))
+    else:
+        _gpu("o", o, shape=(T, H * vd))
+    stride = 0
+    if gates is not None:
+        if not gates.is_cuda or gates.dtype != torch.float32 or gates.dim() != 2 or gates.shape[0] != T or gates.shape[1] < H \
+                or gates.stride(1) != 1:
+            raise KernelError(f"head_mix_gate: gates must be float32 [{T}, >= {H}] on the GPU, got {tuple(gates.shape)} {gates.dtype}")
+        stride = gates.stride(0)
+    _check(load("attention").tuff_head_mix_gate(
+        o.data_ptr(), _dt(o), None if talk is None else talk.data_ptr(), None if gates is None else gates.data_ptr(), stride,
+        out.data_ptr(), _dt(out), T, H, Hkv, vd, _stream()), "head_mix_gate")
+
+
+# ------------------------------------------------- sublayers normed before they join the stream
+def post_norm_add(x, *, y=None, w=None, eps: float = 0.0, mult: float = 1.0, extra=None, next_w=None, next_eps: float = 0.0,
+                  h_out=None, clear_y: bool = False) -> None:
+    """One kernel over the residual stream x (float32 [T, d], in place).  With y float32 [T, d] and w float32 [d]:
+    x <- x + mult * y / sqrt(mean(y^2) + eps) * w (y is then cleared, if asked).  With extra float32 [T, d]:
+    x <- x + extra.  With next_w float32 [d] and h_out [T, d]: h_out = x / sqrt(mean(x^2) + next_eps) * next_w,
+    from the new x."""
+    T, d = x.shape
+    _gpu("x", x, torch.float32, (T, d))
+    _opt("y", y, torch.float32, (T, d))
+    if y is not None:
+        _gpu("w", w, torch.float32, (d,))
+    _opt("extra", extra, torch.float32, (T, d))
+    if (next_w is None) != (h_out is None):
+        raise KernelError("post_norm_add: next_w and h_out go together")
+    if next_w is not None:
+        _gpu("next_w", next_w, torch.float32, (d,))
+        _gpu("h_out", h_out, shape=(T, d))
+    _check(load("postnorm").tuff_post_norm_add(
+        x.data_ptr(), None if y is None else y.data_ptr(), None if y is None else w.data_ptr(), float(eps), float(mult),
+        None if extra is None else extra.data_ptr(), None if next_w is None else next_w.data_ptr(), float(next_eps),
+        None if h_out is None else h_out.data_ptr(), DT_F32 if h_out is None else _dt(h_out), T, d, int(clear_y), _stream()),
+        "post_norm_add")
+
+
+def normed_mean2(a, wa, b, wb, out, *, eps: float, coef: float = 0.5) -> None:
+    """out <- out + coef * (a / sqrt(mean(a^2) + eps) * wa + b / sqrt(mean(b^2) + eps) * wb); a, b, out float32
+    [T, d]; wa, wb float32 [d]."""
+    T, d = a.shape
+    _check(load("postnorm").tuff_normed_mean2(
+        _gpu("a", a, torch.float32, (T, d)), _gpu("wa", wa, torch.float32, (d,)), _gpu("b", b, torch.float32, (T, d)),
+        _gpu("wb", wb, torch.float32, (d,)), float(eps), float(coef), _gpu("out", out, torch.float32, (T, d)), T, d, _stream()),
+        "normed_mean2")
 
 
 ATTN_GENERAL_MAX_DIM = 640   # widest key or value row of the general attention kernel
@@ -1339,14 +1422,32 @@ def delta_scan(q, k, v, a, dt_bias, A_log, b, state, out, *, q_start, q_len, sta
         _gpu("state_slot", state_slot, torch.int32, (R,)), T, R, H, Hk, D, Dv, ld, ldv, _stream()), "delta_scan")
 
 
+def forget_scan(x, bias, lower, state, out, *, q_start, q_len, state_slot, H, D, Dv) -> None:
+    """The forget-gate recurrence over each request's tokens of the step, from and to state[slot] (float32
+    [slots, H, D, Dv]): f = lower + (1 - lower) sigmoid(z + bias); S = diag(f) S + (1 - f) v^T; o = S^T silu(q).
+    x [T, 2 H D + H Dv]: a token's projected rows q, z, v side by side; bias (or None) and lower float32 [H * D];
+    out float32 [T, H * Dv]."""
+    T = x.shape[0]
+    R = q_start.shape[0]
+    if D > SCAN_MAX_DIM:
+        raise KernelError(f"forget_scan: key size {D} above {SCAN_MAX_DIM}")
+    work = torch.empty(2, T, H * D, dtype=torch.float32, device=x.device)       # silu(q) and the gates
+    _check(load("recurrent").tuff_forget_scan(
+        _gpu("x", x, shape=(T, 2 * H * D + H * Dv)), _dt(x), x.shape[1], _opt("bias", bias, torch.float32, (H * D,)),
+        _gpu("lower", lower, torch.float32, (H * D,)), work[0].data_ptr(), work[1].data_ptr(),
+        _gpu("state", state, torch.float32, (None, H, D, Dv)), _gpu("out", out, torch.float32, (T, H * Dv)),
+        _gpu("q_start", q_start, torch.int32, (R,)), _gpu("q_len", q_len, torch.int32, (R,)),
+        _gpu("state_slot", state_slot, torch.int32, (R,)), T, R, H, D, Dv, _stream()), "forget_scan")
+
+
 def head_norm_gate(o, w, gate, out, *, H, Dv, eps, per_head_weight: bool, gate_activation: Optional[str]) -> None:
     """out[t, h] = o[t, h] / sqrt(mean(o[t, h]^2) + eps) * w * f(gate[t, h]); o float32 [T, H * Dv]; w float32
     [H * Dv] (per_head_weight) or [Dv] (shared by the heads); out [T, H * Dv] of the compute type, gate of that
-    type or float32."""
+    type or float32, or None for no gate."""
     T = o.shape[0]
     _check(load("recurrent").tuff_head_norm_gate(
         _gpu("o", o, torch.float32, (T, H * Dv)), _gpu("w", w, torch.float32, (H * Dv if per_head_weight else Dv,)),
-        Dv if per_head_weight else 0, _gpu("gate", gate, shape=(T, H * Dv)), _dt(gate), _dt(out),
+        Dv if per_head_weight else 0, _opt("gate", gate, shape=(T, H * Dv)), _dt(out if gate is None else gate), _dt(out),
         {None: 0, "silu": 1, "sigmoid": 2}[gate_activation], _gpu("out", out, shape=(T, H * Dv)), T, H, Dv, float(eps), _stream()),
         "head_norm_gate")
 

@@ -1,0 +1,93 @@
+// Kernels of layers that norm a sublayer's output before it joins the residual stream, all in float32.
+//
+// tuff_post_norm_add, a workgroup a token:
+//     x <- x + mult * y / sqrt(mean(y^2) + eps) * w  [+ extra]        (y is then cleared, if asked)
+//     h  = x / sqrt(mean(x^2) + eps_next) * w_next                     (if asked: the next sublayer's input)
+// One launch where a norm, a residual sum, another sum and the next norm would be four.  Without y only the
+// sum with `extra` and the next norm run.  The weights come in as float32 with any offset already added.
+//
+// tuff_normed_mean2, a workgroup a token:
+//     out <- out + coef * (a / sqrt(mean(a^2) + eps) * wa + b / sqrt(mean(b^2) + eps) * wb)
+// for a mixer made of two mixers side by side whose outputs are each normed over the width.
+//
+// Every row's sums run over the row in one fixed order (a thread's elements in ascending order, the
+// butterfly of a wave, the waves in order), so a row's result does not depend on what else is in the step.
+#include "common.h"
+#include <math.h>
+
+namespace {
+constexpr int PN_THREADS = 256;
+constexpr int PN_WAVES = PN_THREADS / WAVE;
+
+template <typename T>
+__global__ __launch_bounds__(PN_THREADS) void post_norm_add_kernel(
+    float* __restrict__ x, float* __restrict__ y, const float* __restrict__ w, float eps, float mult,
+    const float* __restrict__ extra, const float* __restrict__ w_next, float eps_next, T* __restrict__ h_out,
+    int d, int clear_y) {
+    __shared__ float scratch[PN_WAVES];
+    const long long row = (long long)blockIdx.x * d;
+    float* xr = x + row;
+    float inv = 0.f;
+    if (y) {
+        const float* yr = y + row;
+        float ss = 0.f;
+        for (int c = threadIdx.x; c < d; c += PN_THREADS) ss = fmaf(yr[c], yr[c], ss);
+        ss = block_sum<PN_WAVES>(ss, scratch);
+        inv = mult / sqrtf(ss / (float)d + eps);
+    }
+    float ss2 = 0.f;
+    for (int c = threadIdx.x; c < d; c += PN_THREADS) {
+        float v = xr[c];
+        if (y) {
+            v = fmaf(y[row + c] * inv, w[c], v);
+            if (clear_y) y[row + c] = 0.f;
+        }
+        if (extra) v += extra[row + c];
+        if (y || extra) xr[c] = v;
+        ss2 = fmaf(v, v, ss2);
+    }
+    if (!h_out) return;
+    ss2 = block_sum<PN_WAVES>(ss2, scratch);
+    const float inv2 = 1.0f / sqrtf(ss2 / (float)d + eps_next);
+    // (a thread reads back the elements it wrote itself)
+    for (int c = threadIdx.x; c < d; c += PN_THREADS) h_out[row + c] = from_f32<T>(xr[c] * inv2 * w_next[c]);
+}
+
+__global__ __launch_bounds__(PN_THREADS) void normed_mean2_kernel(
+    const float* __restrict__ a, const float* __restrict__ wa, const float* __restrict__ b, const float* __restrict__ wb,
+    float eps, float coef, float* __restrict__ out, int d) {
+    __shared__ float scratch[PN_WAVES];
+    const long long row = (long long)blockIdx.x * d;
+    float sa = 0.f, sb = 0.f;
+    for (int c = threadIdx.x; c < d; c += PN_THREADS) {
+        sa = fmaf(a[row + c], a[row + c], sa);
+        sb = fmaf(b[row + c], b[row + c], sb);
+    }
+    sa = block_sum<PN_WAVES>(sa, scratch);
+    sb = block_sum<PN_WAVES>(sb, scratch);
+    const float ia = 1.0f / sqrtf(sa / (float)d + eps), ib = 1.0f / sqrtf(sb / (float)d + eps);
+    for (int c = threadIdx.x; c < d; c += PN_THREADS)
+        out[row + c] += coef * (a[row + c] * ia * wa[c] + b[row + c] * ib * wb[c]);
+}
+}  // namespace
+
+// x float32 [T][d] in place; y float32 [T][d] or null; w float32 [d] (with y); extra float32 [T][d] or null;
+// w_next float32 [d] and h_out [T][d] of type out_dt, or both null.
+TUFF_EXPORT int tuff_post_norm_add(float* x, float* y, const float* w, float eps, float mult, const float* extra,
+                                   const float* w_next, float eps_next, void* h_out, int out_dt, int n_tokens, int d,
+                                   int clear_y, hipStream_t stream) {
+    if (n_tokens <= 0) return 0;
+    if (d <= 0 || (y && !w) || ((w_next == nullptr) != (h_out == nullptr))) return -2;
+    dim3 grid(n_tokens), block(PN_THREADS);
+    if (out_dt == DT_F32) hipLaunchKernelGGL(post_norm_add_kernel<float>, grid, block, 0, stream, x, y, w, eps, mult, extra, w_next, eps_next, (float*)h_out, d, clear_y);
+    else hipLaunchKernelGGL(post_norm_add_kernel<bf16_t>, grid, block, 0, stream, x, y, w, eps, mult, extra, w_next, eps_next, (bf16_t*)h_out, d, clear_y);
+    return launch_status();
+}
+
+TUFF_EXPORT int tuff_normed_mean2(const float* a, const float* wa, const float* b, const float* wb, float eps, float coef,
+                                  float* out, int n_tokens, int d, hipStream_t stream) {
+    if (n_tokens <= 0) return 0;
+    if (d <= 0) return -2;
+    hipLaunchKernelGGL(normed_mean2_kernel, dim3(n_tokens), dim3(PN_THREADS), 0, stream, a, wa, b, wb, eps, coef, out, d);
+    return launch_status();
+}

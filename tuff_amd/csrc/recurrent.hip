@@ -1,7 +1,7 @@
 // Kernels of mixers that carry a fixed-size state from token to token: the blend of a token's input
 // with the one before it (token shift), a short causal convolution per channel with an activation,
-// and two matrix-state recurrences, a decaying outer-product memory with a bonus for the current
-// token ("wkv") and a gated delta rule.  States are float32 and live in a slot per request; a step
+// and three matrix-state recurrences, a decaying outer-product memory with a bonus for the current
+// token ("wkv"), a gated delta rule, and a memory whose forget gate also sets the write strength.  States are float32 and live in a slot per request; a step
 // brings each request's next tokens (one decoded token or a portion of a prompt of any length),
 // tokens flat and ordered by request, and every kernel continues from the slot and leaves it ready
 // for the next step.  The recurrences run token by token in one fixed order of operations, so a
@@ -122,6 +122,7 @@ __global__ void conv_state_kernel(const T* __restrict__ x, float* __restrict__ s
 //
 // wkv:    o_j = sum_i r_i S_ij + bonus v_j;   S_ij <- w_i S_ij + k_i v_j
 // delta:  S_ij <- g_i S_ij;  e_j = beta (v_j - sum_i k_i S_ij);  S_ij <- S_ij + k_i e_j;  o_j = sum_i q_i S_ij
+// forget: S_ij <- f_i S_ij + (1 - f_i) v_j;  o_j = sum_i q_i S_ij      (the read sees the token's own write; no key)
 struct PrepArgs {
     const void *a, *k;              // r or q, k: rows of Ha*D of the compute type, lda apart
     float* decay;                   // in: lw or a [T][H*D]; out, in place: w or g
@@ -170,6 +171,20 @@ __global__ __launch_bounds__(WAVE) void scan_prep_kernel(PrepArgs p) {
     }
 }
 
+// What enters the forget-gate recurrence: x holds a token's projected rows [q (H*D) | z (H*D) | ...], ld apart;
+// qn = silu(q) and f = lower + (1 - lower) sigmoid(z + bias), both float32 [T][H*D].
+template <typename T>
+__global__ void forget_prep_kernel(const T* __restrict__ x, long long ld, const float* __restrict__ bias,
+                                   const float* __restrict__ lower, float* __restrict__ qn, float* __restrict__ f, int HD) {
+    const long long t = blockIdx.x;
+    const T* row = x + t * ld;
+    for (int c = blockIdx.y * blockDim.x + threadIdx.x; c < HD; c += gridDim.y * blockDim.x) {
+        const float lo = lower[c];
+        qn[t * HD + c] = siluf_(to_f32(row[c]));
+        f[t * HD + c] = lo + (1.0f - lo) * sigmoidf_(to_f32(row[HD + c]) + (bias ? bias[c] : 0.f));
+    }
+}
+
 struct ScanArgs {
     const void *a, *k, *v;          // per token: a (r, or unit q) and k [T][Ha*D]; v: rows of H*Dv, ldv apart   (Ha: heads of a and k)
     const float* decay;             // per token [T][H*D]: w or g
@@ -201,7 +216,8 @@ __device__ __forceinline__ float group_sum(float v) {
 }
 
 // TA: type of a and k (the compute type for wkv's r and k, float for the delta rule's unit vectors); T: type of v.
-template <typename TA, typename T, int NI16, int SPLIT, bool DELTA>
+// FORGET: a holds silu(q) in float32, the decay is the forget gate f and the key is 1 - f (k and scalar are not used).
+template <typename TA, typename T, int NI16, int SPLIT, bool DELTA, bool FORGET = false>
 __global__ __launch_bounds__(WAVE) void scan_kernel(ScanArgs p) {
     constexpr int RP = NI16 * 4;                       // rows of the state's column a lane keeps
     constexpr int DP = RP * SPLIT;                     // key channels, padded
@@ -299,13 +315,18 @@ __global__ __launch_bounds__(WAVE) void scan_kernel(ScanArgs p) {
                 const f32x4 r4 = *(const f32x4*)&sa[tt][row0 + g4 * 4];
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
-                    o4[e] = fmaf(r4[e], s[g4 * 4 + e], o4[e]);
-                    s[g4 * 4 + e] = fmaf(w4[e], s[g4 * 4 + e], k4[e] * vt);
+                    if (FORGET) {
+                        s[g4 * 4 + e] = fmaf(w4[e], s[g4 * 4 + e], k4[e] * vt);
+                        o4[e] = fmaf(r4[e], s[g4 * 4 + e], o4[e]);
+                    } else {
+                        o4[e] = fmaf(r4[e], s[g4 * 4 + e], o4[e]);
+                        s[g4 * 4 + e] = fmaf(w4[e], s[g4 * 4 + e], k4[e] * vt);
+                    }
                 }
             }
         }
         float o = group_sum<SPLIT>((o4[0] + o4[1]) + (o4[2] + o4[3]));
-        if (!DELTA) o = fmaf(sc, vt, o);
+        if (!DELTA && !FORGET) o = fmaf(sc, vt, o);
         // (the lanes of a group hold the same sum and write it to the same place: no lane is switched off for it)
         if (jv) orow[(unsigned)tt * (unsigned)(H * Dv)] = o;
     };
@@ -322,7 +343,11 @@ __global__ __launch_bounds__(WAVE) void scan_kernel(ScanArgs p) {
             for (int e = 0; e < PER; ++e) {
                 const int i = lane + e * WAVE;
                 const bool ok = i < D;                 // (tokens beyond the chunk's last are staged and never read)
-                if (i < DP) { sa[tt][i] = ok ? to_f32(fa[tt][e]) : 0.f; sk[tt][i] = ok ? to_f32(fk[tt][e]) : 0.f; sw[tt][i] = ok ? fw[tt][e] : 0.f; }
+                if (i < DP) {
+                    sa[tt][i] = ok ? to_f32(fa[tt][e]) : 0.f;
+                    sk[tt][i] = ok ? (FORGET ? 1.0f - fw[tt][e] : to_f32(fk[tt][e])) : 0.f;
+                    sw[tt][i] = ok ? fw[tt][e] : 0.f;
+                }
             }
         }
         if (c0 + CH < n) fetch(t0 + c0 + CH, min(CH, n - c0 - CH));
@@ -349,7 +374,7 @@ __global__ __launch_bounds__(WAVE) void scan_kernel(ScanArgs p) {
 
 // ---------------------------------------------------------- per-head unit norm, weight and gate
 // y[t][h][j] = o[t][h][j] / sqrt(mean_j o^2 + eps) * w[(h * w_stride) + j] * f(gate[t][h][j]);
-// f: 0 identity, 1 silu, 2 sigmoid.  A wave per (token, head).
+// f: 0 identity, 1 silu, 2 sigmoid; without a gate the factor is 1.  A wave per (token, head).
 template <typename TG, typename T>
 __global__ __launch_bounds__(WAVE) void head_norm_gate_kernel(const float* __restrict__ o, const float* __restrict__ w, int w_stride,
                                                               const TG* __restrict__ gate, int gate_fn, T* __restrict__ y,
@@ -361,14 +386,14 @@ __global__ __launch_bounds__(WAVE) void head_norm_gate_kernel(const float* __res
     ss = wave_sum(ss);
     const float inv = 1.0f / sqrtf(ss / (float)Dv + eps);
     for (int j = threadIdx.x; j < Dv; j += WAVE) {
-        float g = to_f32(gate[row * Dv + j]);
+        float g = gate ? to_f32(gate[row * Dv + j]) : 1.f;
         if (gate_fn == 1) g = siluf_(g);
         else if (gate_fn == 2) g = sigmoidf_(g);
         y[row * Dv + j] = from_f32<T>(src[j] * inv * w[(long long)blockIdx.y * w_stride + j] * g);
     }
 }
 
-template <typename TA, typename T, bool DELTA>
+template <typename TA, typename T, bool DELTA, bool FORGET = false>
 int launch_scan(const ScanArgs& p, int R, hipStream_t stream) {
     if (p.H > 65535 || p.D > 256) return -2;
     const bool narrow = p.D <= 32;                      // four lanes a value channel; else sixteen
@@ -376,7 +401,7 @@ int launch_scan(const ScanArgs& p, int R, hipStream_t stream) {
     const int ni = narrow ? (p.D + 15) / 16 : (p.D + 63) / 64;
     dim3 grid(R, p.H, ceil_div(p.Dv, WAVE / split)), block(WAVE);
     if (grid.z > 65535) return -2;
-#define SCAN(NI, SPLIT) hipLaunchKernelGGL((scan_kernel<TA, T, NI, SPLIT, DELTA>), grid, block, 0, stream, p)
+#define SCAN(NI, SPLIT) hipLaunchKernelGGL((scan_kernel<TA, T, NI, SPLIT, DELTA, FORGET>), grid, block, 0, stream, p)
     if (narrow) { if (ni <= 1) SCAN(1, 4); else SCAN(2, 4); }
     else if (ni <= 1) SCAN(1, 16);
     else if (ni <= 2) SCAN(2, 16);
@@ -467,4 +492,24 @@ TUFF_EXPORT int tuff_head_norm_gate(const float* o, const float* w, int w_stride
     else if (dt == DT_BF16) hipLaunchKernelGGL((head_norm_gate_kernel<bf16_t, bf16_t>), grid, block, 0, stream, o, w, w_stride, (const bf16_t*)gate, gate_fn, (bf16_t*)y, H, Dv, eps);
     else return -2;
     return launch_status();
+}
+
+// forget: x rows [q (H*D) | z (H*D) | v (H*Dv)] of type dt, ld elements apart, as projected; bias (or null) and lower
+// float32 [H*D]; work arrays qn, f float32 [T][H*D]; state float32 [slots][H][D][Dv]; out float32 [T][H][Dv].
+TUFF_EXPORT int tuff_forget_scan(const void* x, int dt, long long ld, const float* bias, const float* lower, float* qn, float* f,
+                                 float* state, float* out, const int* q_start, const int* q_len, const int* state_slot,
+                                 int n_tokens, int n_requests, int H, int D, int Dv, hipStream_t stream) {
+    if (n_requests <= 0 || n_tokens <= 0) return 0;
+    if (H <= 0 || H > 65535 || ld < 2LL * H * D + (long long)H * Dv) return -2;
+    const int HD = H * D;
+    dim3 grid(n_tokens, ceil_div(HD, 256)), block(256);
+    if (dt == DT_F32) hipLaunchKernelGGL(forget_prep_kernel<float>, grid, block, 0, stream, (const float*)x, ld, bias, lower, qn, f, HD);
+    else hipLaunchKernelGGL(forget_prep_kernel<bf16_t>, grid, block, 0, stream, (const bf16_t*)x, ld, bias, lower, qn, f, HD);
+    int rc = launch_status();
+    if (rc != 0) return rc;
+    // (k and the per-token scalar are loaded and not used: they point at arrays of the right reach)
+    const void* v = dt == DT_F32 ? (const void*)((const float*)x + 2LL * HD) : (const void*)((const bf16_t*)x + 2LL * HD);
+    ScanArgs p{qn, qn, v, f, f, state, out, q_start, q_len, state_slot, H, H, D, Dv, ld};
+    return dt == DT_F32 ? launch_scan<float, float, false, true>(p, n_requests, stream)
+                        : launch_scan<float, bf16_t, false, true>(p, n_requests, stream);
 }

@@ -18,6 +18,7 @@ class LayerRun:
     block: int                      # index into DecoderModel.blocks
     cache: Optional[int] = None     # cache entry this run uses (default: one of its own)
     writes: bool = True             # False: only reads the entry, which an earlier run writes
+    reinject: bool = False          # True: the embedding (as it entered the first run) is added to x before this run
 
 
 class _Head:
@@ -50,6 +51,9 @@ class DecoderModel:
             raise ValueError("a model with several residual streams needs at least one and blocks that take them")
         if self.streams is None and any(getattr(b, "multi_stream", False) for b in blocks):
             raise ValueError("a block over several residual streams in a model that keeps one")
+        #: every block hands the next one its first normed input (Block.carries_norm): the kernel that adds a block's
+        #: last output into the stream also reads the stream for whoever comes next
+        self.carries = bool(blocks) and all(getattr(b, "carries_norm", False) for b in blocks)
         #: debugging aid: called as on_layer(run index, x [T, d] or xs [S, T, d]) after every layer run; while it
         #: is set no step is recorded into a graph
         self.on_layer = None
@@ -72,7 +76,7 @@ class DecoderModel:
                     next_id += 1
                 cache = next_id
                 used.add(cache)
-            self.schedule.append(LayerRun(r.block, cache, r.writes))
+            self.schedule.append(LayerRun(r.block, cache, r.writes, r.reinject))
         # Every cache entry has exactly one writer, which comes before its readers.  A run's entry is named
         # by LayerRun.cache; a mixer that declares several things to keep has the entries (cache, 0),
         # (cache, 1), ... in the order of its declarations.
@@ -180,9 +184,18 @@ class DecoderModel:
             return self._finish(x, ctx, False, False)
         x = torch.empty(ctx.T, self.hidden_size, dtype=torch.float32, device=rt.device)
         ops.embed_rows(self.embedding, ctx.tokens, x, self.embedding_scale)
+        x0 = None
+        if any(r.reinject for r in self.schedule):
+            # the embedding as it entered the first run, for the runs before which it joins the stream again
+            x0 = torch.empty_like(x)
+            ops.embed_rows(self.embedding, ctx.tokens, x0, self.embedding_scale)
+        if self.carries:
+            return self._finish(self._forward_carry(x, x0, ctx, cache_views), ctx, False, False)
         head_fused, all_rows = self._head_fused(ctx)
         for i, run in enumerate(self.schedule):
             block = self.blocks[run.block]
+            if run.reinject:
+                ops.post_norm_add(x, extra=x0)
             if getattr(block, "takes_next_norm", False):
                 if i + 1 < len(self.schedule):
                     nb = self.blocks[self.schedule[i + 1].block]
@@ -195,6 +208,32 @@ class DecoderModel:
             if self.on_layer is not None:
                 self.on_layer(i, x)
         return self._finish(x, ctx, head_fused, all_rows)
+
+    def _forward_carry(self, x, x0, ctx, cache_views) -> torch.Tensor:
+        """The layers of a model whose blocks hand each other their first normed input.  The kernel that adds a block's
+        last output into x also adds the embedding where the next run takes it again, and norms x for the next block;
+        the final norm runs with the head, on the wanted rows."""
+        last = len(self.schedule) - 1
+        y = torch.empty(ctx.T, self.hidden_size, dtype=torch.float32, device=self.rt.device)
+        ops.fill_u32(y, 0)
+        carry = None
+        for i, run in enumerate(self.schedule):
+            block = self.blocks[run.block]
+            nxt = self.schedule[i + 1] if i < last else None
+            extra = x0 if nxt is not None and nxt.reinject else None
+            if run.reinject and carry is None:
+                ops.post_norm_add(x, extra=x0)              # (nobody before this run could add it)
+            if self.on_layer is not None and extra is not None:
+                # the hook sees x as the layer leaves it: the embedding joins afterwards, in a launch of its own
+                block.forward(x, ctx, self._views_of(i, cache_views), run.writes, carry=carry, next_read=None, y=y)
+                self.on_layer(i, x)
+                carry = None
+                continue
+            read = self.blocks[nxt.block].first_read() if nxt is not None else None
+            carry = block.forward(x, ctx, self._views_of(i, cache_views), run.writes, carry=carry, next_read=read, y=y, extra=extra)
+            if self.on_layer is not None:
+                self.on_layer(i, x)
+        return x
 
     def _forward_streams(self, ctx, cache_views) -> torch.Tensor:
         """The layers over several residual streams; returns the sum of the streams, float32 [T, d].  The kernel that

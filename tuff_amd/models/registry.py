@@ -74,6 +74,9 @@ def _register_builtin() -> None:
     from ..config.kugalorn import KugalornConfig
     from .kugalorn import build_kugalorn
     register_architecture(KugalornConfig.architecture, KugalornConfig, build_kugalorn)
+    from ..config.loluzen import LoluzenConfig
+    from .loluzen import build_loluzen
+    register_architecture(LoluzenConfig.architecture, LoluzenConfig, build_loluzen)
 
 
 _register_builtin()

@@ -6,7 +6,11 @@ at the token's slot; every token attends to the cached keys of its request up to
 position (within `window` if given); query head i reads kv head i // (H / Hkv); scores are
 scaled by 1/sqrt(hd); o = W_o concat(heads).  Options: a per-head norm of q and k without a
 weight (unit root mean square), and a distance penalty slope_h * (i - j) taken off the scaled
-score of query i and key j, slope_h = 2^(-span (h + 1) / H).
+score of query i and key j, slope_h = 2^(-span (h + 1) / H).  Further options: biases on q, k, v; a
+logarithmic distance penalty r1_h ln(1 + r2_h (i - j)) with learned r1, r2 per head; the heads' softmax
+weights mixed by a learned [H, H] matrix, p'_h = sum_g talk[h, g] p_g, head h applying p'_h to the values of
+its own kv head; a short causal convolution per channel on q, k and v right after the projection (its last
+taps - 1 inputs are state of the request); a gate per head, sigmoid(W_g h)_h, on the head's output.
 Reference: src/lfm25_engine.c:386-405, src/lfm25_gpu.cu:420-485, :506-558.
 """
 from __future__ import annotations
@@ -18,14 +22,17 @@ import numpy as np
 import torch
 
 from ..csrc import ops
-from .base import MIXERS, Mixer, PagedKV, PositionEncoding, Runtime, WeightDecl
+from .base import MIXERS, FixedState, Mixer, PagedKV, PositionEncoding, Runtime, WeightDecl
 from .linear import Linear
 
 
 class PagedAttention:
     """Which attention kernels run over a paged cache, and their launch: shared by the mixers whose attention is
     softmax(q . k * scale [- slope (i - j)]) over a request's cached positions (all of them or a window), with
-    grouped heads and optional sinks.  It reads the mixer's H, Hkv, hd, vd, window, scale, sinks, slopes."""
+    grouped heads and optional sinks.  It reads the mixer's H, Hkv, hd, vd, window, scale, sinks, slopes and, where
+    the mixer has them, log_distance ((r1, r2): the penalty r1_h ln(1 + r2_h (i - j))) and talk (a matrix that mixes
+    the heads' softmax weights: o is then float32 [T, H * Hkv * vd], every head's weights on every kv head's values,
+    from which ops.head_mix_gate forms the mixed heads)."""
 
     @staticmethod
     def _upload(array, device):
@@ -69,6 +76,14 @@ class PagedAttention:
 
     def attend(self, q, o, ctx, cache, g) -> None:
         G = self.H // self.Hkv
+        log_distance, talk = getattr(self, "log_distance", None), getattr(self, "talk", None)
+        if log_distance is not None or talk is not None:
+            ops.attention_general(q, cache.k, cache.v, o, block_table=g.block_table,
+                                  req_of_token=ctx.req_of_token, positions=ctx.positions,
+                                  H=self.H, Hkv=self.Hkv, hd=self.hd, page_size=cache.page_size,
+                                  window=self.window or 0, scale=self.scale, vd=self.vd, sinks=self.sinks, slopes=self.slopes,
+                                  log_distance=log_distance, all_values=talk is not None)
+            return
         if self.vd == self.hd and ops.attention_mfma_supported(q.dtype, self.hd, cache.page_size):
             common = dict(block_table=g.block_table, req_info=ctx.req_info, H=self.H, Hkv=self.Hkv, hd=self.hd,
                           page_size=cache.page_size, max_ctx_len=ctx.max_ctx_len, window=self.window or 0,
@@ -108,11 +123,14 @@ class AttentionMixer(Mixer, PagedAttention):
                  names: dict[str, str], qk_norm_eps: Optional[float] = None,
                  position: Optional[PositionEncoding] = None, window: Optional[int] = None,
                  scale: Optional[float] = None, aliases: Optional[dict[str, tuple]] = None,
-                 value_dim: Optional[int] = None, slope_span: Optional[float] = None):
+                 value_dim: Optional[int] = None, slope_span: Optional[float] = None, conv_taps: int = 1):
         """names: checkpoint names of 'q', 'k', 'v', 'o' and, with qk_norm_eps, 'q_norm', 'k_norm' (without these
         two names the norm has no weight: q and k are divided by their root mean square over the head); with a
         'sink' among them the heads have sinks.  value_dim: width of a value head (default: head_dim).
-        slope_span: heads have distance slopes 2^(-slope_span (h + 1) / H) (None: none)."""
+        slope_span: heads have distance slopes 2^(-slope_span (h + 1) / H) (None: none).
+        Further names switch further options on: 'q.b', 'k.b', 'v.b' biases of the projections; 'r1', 'r2' [H] the
+        logarithmic distance penalty; 'talk' [H, H] the matrix that mixes the heads' softmax weights; 'g' [H, d] the
+        gate per head; with conv_taps > 1, 'q.conv', 'k.conv', 'v.conv' [channels, taps] the convolutions' taps."""
         if num_heads % num_kv_heads:
             raise ValueError(f"heads {num_heads} must be a multiple of kv heads {num_kv_heads}")
         if head_dim > 256:
@@ -121,8 +139,8 @@ class AttentionMixer(Mixer, PagedAttention):
         self.vd = self.hd if value_dim is None else int(value_dim)
         if self.vd > 256 or self.vd < 1:
             raise ValueError(f"value size {self.vd} is outside 1..256")
-        if self.vd != self.hd and position is not None:
-            raise ValueError("values of another width than keys go with no position encoding")
+        if self.vd != self.hd and position is not None and position.rotary_tables() is None:
+            raise ValueError("values of another width than keys go with a rotary encoding or none")
         self.has_sink = "sink" in names
         self.norm_has_weight = qk_norm_eps is not None and "q_norm" in names
         self.slope_span = None if slope_span is None else float(slope_span)
@@ -133,9 +151,18 @@ class AttentionMixer(Mixer, PagedAttention):
         self.scale = float(scale) if scale is not None else 1.0 / math.sqrt(self.hd)
         self.names = dict(names)
         al = aliases or {}
+        self.has_bias = "q.b" in names
+        self.has_log_distance, self.has_talk = "r1" in names, "talk" in names
+        self.K = int(conv_taps)
+        if not 1 <= self.K <= ops.CONV_ACT_MAX_TAPS:
+            raise ValueError(f"{self.K} convolution taps are outside 1..{ops.CONV_ACT_MAX_TAPS}")
+        self.C = (self.H + self.Hkv) * self.hd + self.Hkv * self.vd            # channels of a token's q, k, v
+        self.log_distance = self.talk = self.taps = None
         self.qkv = Linear([names["q"], names["k"], names["v"]], self.d,
                           [self.H * self.hd, self.Hkv * self.hd, self.Hkv * self.vd],
-                          aliases=[al.get("q", ()), al.get("k", ()), al.get("v", ())])
+                          aliases=[al.get("q", ()), al.get("k", ()), al.get("v", ())],
+                          bias=[names["q.b"], names["k.b"], names["v.b"]] if self.has_bias else None)
+        self.gate = Linear(names["g"], self.d, self.H) if "g" in names else None
         self.out = Linear(names["o"], self.H * self.vd, self.d, aliases=[al.get("o", ())])
         self._al = al
         self.q_norm_w = self.k_norm_w = None
@@ -157,10 +184,21 @@ class AttentionMixer(Mixer, PagedAttention):
             decls += self.position.weight_decls()
         if self.has_sink:
             decls.append(WeightDecl(self.names["sink"], (self.H,), "normal", aliases=self._al.get("sink", ())))
+        if self.has_log_distance:
+            decls += [WeightDecl(self.names["r1"], (self.H,), "norm"), WeightDecl(self.names["r2"], (self.H,), "norm")]
+        if self.has_talk:
+            decls.append(WeightDecl(self.names["talk"], (self.H, self.H), "identity"))
+        if self.gate is not None:
+            decls += self.gate.weight_decls()
+        if self.K > 1:
+            decls += [WeightDecl(self.names[k + ".conv"], (n, self.K), "normal")
+                      for k, n in (("q", self.H * self.hd), ("k", self.Hkv * self.hd), ("v", self.Hkv * self.vd))]
         return decls
 
     def kernel_modules(self):
         mods = ["rope_kv", "attention", "attention_mfma", "attention_prefill"]
+        if self.K > 1:
+            mods.append("recurrent")
         if self.position is not None:
             mods += self.position.kernel_modules()
         return mods
@@ -169,7 +207,9 @@ class AttentionMixer(Mixer, PagedAttention):
         return self.position.token_inputs() if self.position is not None else []
 
     def cache_spec(self):
-        return PagedKV(self.Hkv, self.hd, self.window, value_dim=None if self.vd == self.hd else self.vd)
+        kv = PagedKV(self.Hkv, self.hd, self.window, value_dim=None if self.vd == self.hd else self.vd)
+        # with a convolution: its last taps - 1 inputs, then the keys and values
+        return (FixedState((self.K - 1, self.C)), kv) if self.K > 1 else kv
 
     def bind(self, weights, rt: Runtime):
         self.rt = rt
@@ -191,20 +231,40 @@ class AttentionMixer(Mixer, PagedAttention):
             self.position.bind(weights, rt)
         if self.has_sink:
             self.sinks = weights[self.names["sink"]].float().contiguous()
+        f32 = lambda name: weights[self.names[name]].float().contiguous()
+        if self.has_log_distance:
+            self.log_distance = (f32("r1"), f32("r2"))
+        if self.has_talk:
+            self.talk = f32("talk")
+        if self.gate is not None:
+            self.gate.bind(weights, rt)
+        if self.K > 1:
+            self.taps = torch.cat([f32("q.conv"), f32("k.conv"), f32("v.conv")]).contiguous()      # [C, K]
 
     def forward(self, h, ctx, cache, residual, write_cache: bool = True, next_norm=None) -> None:
         T = h.shape[0]
         H, Hkv, hd, vd = self.H, self.Hkv, self.hd, self.vd
         qkv = self.qkv.forward(h)
+        # the gate's activation reads the product's float32 sums
+        gates = self.gate.forward(h, out_dtype=torch.float32) if self.gate is not None else None
+        if self.K > 1:
+            if not write_cache:
+                raise ValueError("a convolution's state has one owner: it cannot be read by another run")
+            tail, cache = cache
+            x, qkv = qkv, self.rt.empty(T, self.C)
+            ops.conv_act(x, self.taps, tail.state, qkv, req_of_token=ctx.req_of_token, q_start=ctx.q_start,
+                         state_slot=ctx.state_slot, q_len=ctx.q_len, activation=None)
         q = self.rt.empty(T, H * hd) if vd == hd else None
-        o = self.rt.empty(T, H * vd)
+        # (with mixed heads: every head's weights on every kv head's values, float32, for the kernel that mixes them)
+        o = self.rt.empty(T, H * vd) if self.talk is None else torch.empty(T, H * Hkv * vd, dtype=torch.float32, device=qkv.device)
         norm = dict(eps=self.eps or 0.0, q_norm_w=self.q_norm_w, k_norm_w=self.k_norm_w)
         tables = self.position.rotary_tables() if self.position is not None else None
         fused = self.position is None or tables is not None
         # a position encoding of its own: norm, then its apply(), then the cache write
         k = None if fused else self.rt.empty(T, Hkv * hd)
 
-        one_kernel = (fused and tables is not None and ctx.max_q_len == 1 and self.sinks is None and ops.attention_decode_fused_supported(
+        one_kernel = (fused and tables is not None and ctx.max_q_len == 1 and self.sinks is None and self.talk is None
+                      and self.log_distance is None and ops.attention_decode_fused_supported(
             qkv.dtype, H, Hkv, hd, cache.page_size, tables[1], tables[2]))
 
         def over_the_cache(ctx):
@@ -212,9 +272,10 @@ class AttentionMixer(Mixer, PagedAttention):
             g = ctx.groups[cache.group]
             if vd != hd:
                 # keys and values of different widths: the rows are cut out (normed, where there is a norm) and written
-                if self.eps is not None:
+                if self.eps is not None or tables is not None:
                     qq, kk = self.rt.empty(T, H * hd), self.rt.empty(T, Hkv * hd)
-                    ops.qkv_post(qkv, qq, H=H, Hkv=Hkv, hd=hd, positions=ctx.positions, k_out=kk, wide_rows=True, **norm)
+                    rot = {} if tables is None else dict(inv_freq=tables[0], rotary_dim=tables[1], interleaved=tables[2])
+                    ops.qkv_post(qkv, qq, H=H, Hkv=Hkv, hd=hd, positions=ctx.positions, k_out=kk, wide_rows=True, **norm, **rot)
                 else:
                     qq, kk = qkv[:, :H * hd].contiguous(), qkv[:, H * hd:(H + Hkv) * hd].contiguous()
                 if write_cache:
@@ -249,4 +310,8 @@ class AttentionMixer(Mixer, PagedAttention):
             self.attend(q, o, ctx, cache, g)
 
         ctx.run_eagerly(over_the_cache)
+        if self.talk is not None or gates is not None:
+            mixed = self.rt.empty(T, H * vd)
+            ops.head_mix_gate(o, mixed, H=H, Hkv=Hkv, vd=vd, talk=self.talk, gates=gates)
+            o = mixed
         self.out.forward(o, accumulate_into=residual, next_norm=next_norm)

@@ -7,6 +7,9 @@ with the residual stream x in float32.  A feed-forward of None leaves out the se
 ParallelBlock has one norm whose output both sublayers read:
     h = norm(x);  x += mixer(h) + ffn(h)
 
+SandwichBlock norms a sublayer on both sides:
+    x += m * norm1b(mixer(norm1(x)));  x += m * norm2b(ffn(norm2(x)))
+
 HyperConnectionBlock is the pre-norm layer over several residual streams: a sublayer reads a weighted sum
 of the streams and its output goes back into all of them through a mixing matrix.
 """
@@ -136,6 +139,85 @@ class ParallelBlock(Block):
         if self.ffn is not None:
             kw = {"next_norm": None} if self.ffn.adds_once_through_linear else {}
             self.ffn.forward(h, ctx, x, **kw)
+
+
+@BLOCKS.register("sandwich")
+class SandwichBlock(Block):
+    """x <- x + mult * after1(mixer(before1(x))), then x <- x + mult * after2(ffn(before2(x))): every sublayer is
+    normed before and after.  ffn None: the mixer's sublayer alone.  The four norms are RMS norms (they run inside
+    one kernel, ops.post_norm_add, which norms a sublayer's output, adds it into the stream and reads the next
+    sublayer's input with its norm; the next sublayer may be the next block's first, so forward() takes what the
+    block before left (`carry`) and is told who reads next (`next_read`))."""
+    carries_norm = True
+
+    def __init__(self, before1: Norm, mixer: Mixer, after1: Norm, before2: Optional[Norm] = None,
+                 ffn: Optional[FeedForward] = None, after2: Optional[Norm] = None, *, mult: float = 1.0):
+        if not ((before2 is None) == (ffn is None) == (after2 is None)):
+            raise ValueError("before2, ffn and after2 go together")
+        for n in (before1, after1, before2, after2):
+            if n is not None and not isinstance(n, RMSNorm):
+                raise ValueError("the norms of a sandwich block are RMS norms (they run inside the block's kernel)")
+        self.before1, self.mixer, self.after1 = before1, mixer, after1
+        self.before2, self.ffn, self.after2 = before2, ffn, after2
+        self.mult = float(mult)
+
+    def _parts(self):
+        return [p for p in (self.before1, self.mixer, self.after1, self.before2, self.ffn, self.after2) if p is not None]
+
+    @property
+    def graph_safe(self):
+        return all(p.graph_safe for p in self._parts())
+
+    @property
+    def records_portions(self):
+        return all(p.records_portions for p in self._parts())
+
+    def weight_decls(self):
+        return [d for p in self._parts() for d in p.weight_decls()]
+
+    def kernel_modules(self):
+        return ["postnorm", "elementwise"] + [m for p in self._parts() for m in p.kernel_modules()]
+
+    def token_inputs(self):
+        return [t for p in self._parts() for t in p.token_inputs()]
+
+    def bind(self, weights, rt: Runtime):
+        self.rt = rt
+        for p in self._parts():
+            p.bind(weights, rt)
+
+    def first_read(self):
+        """(norm weight float32 [d], eps): what the block before needs to prepare this block's first input."""
+        return self.before1.weight_f32, self.before1.eps
+
+    def forward(self, x, ctx, cache, write_cache: bool = True, carry=None, next_read=None, y=None, extra=None):
+        """x float32 [T, d], in place.  carry: before1(x) where the block before left it (None: computed here).
+        next_read: (norm weight, eps) of whoever reads x next; that norm of the new x is returned (None: nothing is
+        read and None returned).  y: float32 [T, d] of zeros that the sublayers add into (left zero again); None:
+        made here.  extra: float32 [T, d] that joins x after the block's last sublayer, before next_read's norm."""
+        T, d = x.shape
+        if carry is None:
+            carry = self.before1.forward(x)
+        if y is None:
+            y = torch.empty(T, d, dtype=torch.float32, device=x.device)
+            ops.fill_u32(y, 0)
+        kw = {"next_norm": None} if self.mixer.adds_once_through_linear else {}
+        self.mixer.forward(carry, ctx, cache, y, write_cache, **kw)
+        if self.ffn is None:
+            return self._join(x, y, self.after1, next_read, extra)
+        h = self._join(x, y, self.after1, (self.before2.weight_f32, self.before2.eps), None)
+        kw = {"next_norm": None} if self.ffn.adds_once_through_linear else {}
+        self.ffn.forward(h, ctx, y, **kw)
+        return self._join(x, y, self.after2, next_read, extra)
+
+    def _join(self, x, y, after, read, extra):
+        h = None
+        kw = {}
+        if read is not None:
+            h = self.rt.empty(*x.shape)
+            kw = dict(next_w=read[0], next_eps=read[1], h_out=h)
+        ops.post_norm_add(x, y=y, w=after.weight_f32, eps=after.eps, mult=self.mult, extra=extra, clear_y=True, **kw)
+        return h
 
 
 @BLOCKS.register("hyper")

@@ -1,6 +1,7 @@
 """Feed-forwards.
 
 GatedMLP: W_down (act(W_gate h + b_g) * (W_up h + b_u)) + b_d with act silu or the tanh form of gelu, biases optional.
+DenseMLP: W_down act(W_up h + b_u) + b_d without a gate, act the square of relu or any other of the row activations.
 MoE: routed experts W_down act(W_up x) chosen per token by a router, and an optional shared expert.
 
 SwiGLU feed-forward: W_down (silu(W_gate h) * (W_up h)), silu(g) = g / (1 + exp(-g)).
@@ -133,6 +134,62 @@ class GatedMLP(FeedForward):
         gu = self.gate_up.forward(h, out_dtype=torch.float32)       # the activation reads the sums as they are, plus the biases
         act = self.rt.empty(h.shape[0], self.width)
         ops.glu(gu, act, self.activation, self.gu_bias, limit=self.limit, alpha=self.alpha)
+        self.down.forward(act, accumulate_into=residual, next_norm=next_norm)
+
+
+@FEED_FORWARDS.register("dense")
+class DenseMLP(FeedForward):
+    """W_down act(W_up h + b_up) + b_down: no gate.  activation: "relu2" (the square of relu), "silu", "gelu_tanh",
+    "tanh" or "sigmoid".  names: 'up' [F, d], 'down' [d, F] and, with bias=True, 'up.b' [F], 'down.b' [d]."""
+    graph_safe = True
+    records_portions = True
+    adds_once_through_linear = True
+
+    def __init__(self, hidden_size: int, ffn_dim: int, *, names: dict[str, str], activation: str = "relu2", bias: bool = False):
+        if activation not in ops.ACTIVATIONS:
+            raise ValueError(f"unknown activation '{activation}'")
+        self.d, self.F, self.activation, self.has_bias = int(hidden_size), int(ffn_dim), activation, bool(bias)
+        if activation == "sigmoid" and self.F % 8:
+            raise ValueError("a width that is no multiple of 8 needs an activation with act(0) = 0")
+        self._names = dict(names)
+        self._make(self.F)
+        self._decls = self.up.weight_decls() + self.down.weight_decls()
+        if self.has_bias:
+            self._decls.append(WeightDecl(names["up.b"], (self.F,), "normal"))
+
+    def _make(self, width: int) -> None:
+        n = self._names
+        self.up = Linear(n["up"], self.d, width)                     # (its bias goes into the activation's kernel)
+        self.down = Linear(n["down"], width, self.d, bias=n["down.b"] if self.has_bias else None)
+        self.width = width
+
+    def weight_decls(self):
+        return self._decls
+
+    def kernel_modules(self):
+        return ["elementwise"]
+
+    def bind(self, weights, rt: Runtime):
+        self.rt = rt
+        n = self._names
+        u, dn = weights[n["up"]], weights[n["down"]]
+        if self.F % 8 and u.dtype == torch.bfloat16 and dn.dtype == torch.bfloat16:
+            # zero rows of up (with a zero bias: act(0) = 0) and zero columns of down: the same function
+            pad = -self.F % 8
+            weights = dict(weights)
+            weights[n["up"]] = torch.cat([u, u.new_zeros(pad, self.d)])
+            weights[n["down"]] = torch.cat([dn, dn.new_zeros(self.d, pad)], dim=1).contiguous()
+            if self.has_bias:
+                weights[n["up.b"]] = torch.cat([weights[n["up.b"]], weights[n["up.b"]].new_zeros(pad)])
+            self._make(self.F + pad)
+        self.up.bind(weights, rt)
+        self.down.bind(weights, rt)
+        self.up_bias = weights[n["up.b"]].float().contiguous() if self.has_bias else None
+
+    def forward(self, h, ctx, residual, next_norm=None) -> None:
+        u = self.up.forward(h, out_dtype=torch.float32)          # the activation reads the sums as they are, plus the bias
+        act = self.rt.empty(u.shape[0], self.width)
+        ops.act_rows(u, act, self.activation, bias=self.up_bias)
         self.down.forward(act, accumulate_into=residual, next_norm=next_norm)
 
 

@@ -19,6 +19,14 @@ g = exp(-exp(A_log) * softplus(W_a2 (W_a1 h) + dt_bias)) per head and key channe
 multiplied by a weight [Dv] shared by the heads and by sigmoid(W_g2 (W_g1 h)); W_o adds the result into the
 stream.  State per request: the last taps - 1 inputs of the convolutions and S.
 
+ForgetGateMixer (a gated linear recurrence whose forget gate also sets what is written, as in HGRN2).
+q = silu(W_q h) in H heads of D channels, v = W_v h in H heads of Dv; the forget gate per head and key channel is
+f = lower + (1 - lower) sigmoid(W_f h + b) with a learned lower bound `lower` [H*D].  Per head:
+    S <- diag(f) S + (1 - f) v^T;   o = S^T q
+(there is no key: 1 - f stands in its place; the read sees the current token's write).  Each head's o is normed
+over Dv (RMS norm with a weight [Dv] shared by the heads); W_o adds the result into the stream.  State per
+request: S.
+
 States, decays, write strengths and unit norms are float32 in every mode; the recurrences run token by
 token in one order, so a position's result does not depend on how the sequence was cut into steps.
 """
@@ -221,4 +229,54 @@ class GatedDeltaMixer(Mixer):
         y = self.rt.empty(T, self.Cv)
         ops.head_norm_gate(o, self.norm_w, gate, y, H=self.H, Dv=self.Dv, eps=self.eps, per_head_weight=False,
                            gate_activation="sigmoid")
+        self.out.forward(y, accumulate_into=residual, next_norm=next_norm)
+
+
+@MIXERS.register("forget_gate")
+class ForgetGateMixer(Mixer):
+    graph_safe = True
+    records_portions = True
+    adds_once_through_linear = True
+
+    def __init__(self, hidden_size: int, num_heads: int, key_dim: int, value_dim: int, eps: float, *, names: dict[str, str]):
+        """names: checkpoint names of 'q', 'f' [H*D, d], 'f.b', 'lower' [H*D], 'v' [H*Dv, d], 'norm' [Dv], 'o' [d, H*Dv]."""
+        self.d, self.H, self.D, self.Dv, self.eps = int(hidden_size), int(num_heads), int(key_dim), int(value_dim), float(eps)
+        if self.D > ops.SCAN_MAX_DIM:
+            raise ValueError(f"key size {self.D} above {ops.SCAN_MAX_DIM} is not supported by the recurrence kernels")
+        self.names = dict(names)
+        n, HD = self.names, self.H * self.D
+        # one product for q, the gate's logits and v; its float32 sums go into the recurrence's kernels as they are
+        self.qfv = Linear([n["q"], n["f"], n["v"]], self.d, [HD, HD, self.H * self.Dv])
+        self.out = Linear(n["o"], self.H * self.Dv, self.d)
+
+    def weight_decls(self):
+        n, HD = self.names, self.H * self.D
+        return (self.qfv.weight_decls() + [WeightDecl(n["f.b"], (HD,), "normal"), WeightDecl(n["lower"], (HD,), "around:0.5"),
+                                           WeightDecl(n["norm"], (self.Dv,), "norm")] + self.out.weight_decls())
+
+    def kernel_modules(self):
+        return ["recurrent", "elementwise"]
+
+    def cache_spec(self):
+        return FixedState((self.H, self.D, self.Dv))
+
+    def bind(self, weights, rt: Runtime):
+        self.rt = rt
+        n = self.names
+        self.qfv.bind(weights, rt)
+        self.out.bind(weights, rt)
+        f32 = lambda name: weights[n[name]].float().contiguous()
+        self.f_bias, self.lower, self.norm_w = f32("f.b"), f32("lower"), f32("norm")
+
+    def forward(self, h, ctx, cache, residual, write_cache: bool = True, next_norm=None) -> None:
+        if not write_cache:
+            raise ValueError("a recurrent state has one owner: it cannot be read by another run")
+        T = h.shape[0]
+        x = self.qfv.forward(h, out_dtype=torch.float32)
+        o = torch.empty(T, self.H * self.Dv, dtype=torch.float32, device=x.device)
+        ops.forget_scan(x, self.f_bias, self.lower, cache.state, o, q_start=ctx.q_start, q_len=ctx.q_len,
+                        state_slot=ctx.state_slot, H=self.H, D=self.D, Dv=self.Dv)
+        y = self.rt.empty(T, self.H * self.Dv)
+        ops.head_norm_gate(o, self.norm_w, None, y, H=self.H, Dv=self.Dv, eps=self.eps, per_head_weight=False,
+                           gate_activation=None)
         self.out.forward(y, accumulate_into=residual, next_norm=next_norm)
