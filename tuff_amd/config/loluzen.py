@@ -80,7 +80,7 @@ class LoluzenConfig(ModelConfig):
                 _check_sizes(f"{where}.mixer.right", m.get("right"), RECURRENT_KEYS)
             else:
                 _check_sizes(f"{where}.mixer", m, ATTENTION_KEYS)
-                if not _is_int(m.get("conv", 1)):
+                if m.get("conv") is not None and not _is_int(m["conv"]):
                     raise ConfigError(f"{where}.mixer.conv must be a positive number of taps, got {m.get('conv')!r}")
                 rot = m.get("rot")
                 if rot is not None:

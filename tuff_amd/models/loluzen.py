@@ -54,8 +54,8 @@ def _mixer(cfg: LoluzenConfig, i: int):
                           table_positions=ROTARY_TABLE_POSITIONS)
     names = {k: p + k for k in ("q", "k", "v", "o", "g", "q.conv", "k.conv", "v.conv")}
     names.update(q_norm=p + "q.norm", k_norm=p + "k.norm")
-    taps = int(m.get("conv", 1))
-    if taps <= 1:
+    taps = m.get("conv")
+    if taps is None:
         for k in ("q.conv", "k.conv", "v.conv"):
             names.pop(k)
     return AttentionMixer(d, m["heads"], m["kv_heads"], m["dim"], value_dim=m["vdim"], scale=m["scale"],

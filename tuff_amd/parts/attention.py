@@ -123,14 +123,15 @@ class AttentionMixer(Mixer, PagedAttention):
                  names: dict[str, str], qk_norm_eps: Optional[float] = None,
                  position: Optional[PositionEncoding] = None, window: Optional[int] = None,
                  scale: Optional[float] = None, aliases: Optional[dict[str, tuple]] = None,
-                 value_dim: Optional[int] = None, slope_span: Optional[float] = None, conv_taps: int = 1):
+                 value_dim: Optional[int] = None, slope_span: Optional[float] = None, conv_taps: Optional[int] = None):
         """names: checkpoint names of 'q', 'k', 'v', 'o' and, with qk_norm_eps, 'q_norm', 'k_norm' (without these
         two names the norm has no weight: q and k are divided by their root mean square over the head); with a
         'sink' among them the heads have sinks.  value_dim: width of a value head (default: head_dim).
         slope_span: heads have distance slopes 2^(-slope_span (h + 1) / H) (None: none).
         Further names switch further options on: 'q.b', 'k.b', 'v.b' biases of the projections; 'r1', 'r2' [H] the
         logarithmic distance penalty; 'talk' [H, H] the matrix that mixes the heads' softmax weights; 'g' [H, d] the
-        gate per head; with conv_taps > 1, 'q.conv', 'k.conv', 'v.conv' [channels, taps] the convolutions' taps."""
+        gate per head; with conv_taps, 'q.conv', 'k.conv', 'v.conv' [channels, taps] the convolutions' taps (one tap: a
+        factor per channel and no state)."""
         if num_heads % num_kv_heads:
             raise ValueError(f"heads {num_heads} must be a multiple of kv heads {num_kv_heads}")
         if head_dim > 256:
@@ -153,8 +154,8 @@ class AttentionMixer(Mixer, PagedAttention):
         al = aliases or {}
         self.has_bias = "q.b" in names
         self.has_log_distance, self.has_talk = "r1" in names, "talk" in names
-        self.K = int(conv_taps)
-        if not 1 <= self.K <= ops.CONV_ACT_MAX_TAPS:
+        self.K = 0 if conv_taps is None else int(conv_taps)              # 0: no convolution
+        if conv_taps is not None and not 1 <= self.K <= ops.CONV_ACT_MAX_TAPS:
             raise ValueError(f"{self.K} convolution taps are outside 1..{ops.CONV_ACT_MAX_TAPS}")
         self.C = (self.H + self.Hkv) * self.hd + self.Hkv * self.vd            # channels of a token's q, k, v
         self.log_distance = self.talk = self.taps = None
@@ -190,14 +191,14 @@ class AttentionMixer(Mixer, PagedAttention):
             decls.append(WeightDecl(self.names["talk"], (self.H, self.H), "identity"))
         if self.gate is not None:
             decls += self.gate.weight_decls()
-        if self.K > 1:
+        if self.K >= 1:
             decls += [WeightDecl(self.names[k + ".conv"], (n, self.K), "normal")
                       for k, n in (("q", self.H * self.hd), ("k", self.Hkv * self.hd), ("v", self.Hkv * self.vd))]
         return decls
 
     def kernel_modules(self):
         mods = ["rope_kv", "attention", "attention_mfma", "attention_prefill"]
-        if self.K > 1:
+        if self.K >= 1:
             mods.append("recurrent")
         if self.position is not None:
             mods += self.position.kernel_modules()
@@ -238,7 +239,7 @@ class AttentionMixer(Mixer, PagedAttention):
             self.talk = f32("talk")
         if self.gate is not None:
             self.gate.bind(weights, rt)
-        if self.K > 1:
+        if self.K >= 1:
             self.taps = torch.cat([f32("q.conv"), f32("k.conv"), f32("v.conv")]).contiguous()      # [C, K]
 
     def forward(self, h, ctx, cache, residual, write_cache: bool = True, next_norm=None) -> None:
@@ -247,12 +248,14 @@ class AttentionMixer(Mixer, PagedAttention):
         qkv = self.qkv.forward(h)
         # the gate's activation reads the product's float32 sums
         gates = self.gate.forward(h, out_dtype=torch.float32) if self.gate is not None else None
-        if self.K > 1:
-            if not write_cache:
+        if self.K >= 1:
+            if not write_cache and self.K > 1:
                 raise ValueError("a convolution's state has one owner: it cannot be read by another run")
-            tail, cache = cache
+            tail = None
+            if self.K > 1:
+                tail, cache = cache
             x, qkv = qkv, self.rt.empty(T, self.C)
-            ops.conv_act(x, self.taps, tail.state, qkv, req_of_token=ctx.req_of_token, q_start=ctx.q_start,
+            ops.conv_act(x, self.taps, None if tail is None else tail.state, qkv, req_of_token=ctx.req_of_token, q_start=ctx.q_start,
                          state_slot=ctx.state_slot, q_len=ctx.q_len, activation=None)
         q = self.rt.empty(T, H * hd) if vd == hd else None
         # (with mixed heads: every head's weights on every kv head's values, float32, for the kernel that mixes them)
@@ -310,8 +313,8 @@ class AttentionMixer(Mixer, PagedAttention):
             self.attend(q, o, ctx, cache, g)
 
         ctx.run_eagerly(over_the_cache)
+        heads = o             # (over_the_cache keeps `o` for its replays: the name is not bound anew)
         if self.talk is not None or gates is not None:
-            mixed = self.rt.empty(T, H * vd)
-            ops.head_mix_gate(o, mixed, H=H, Hkv=Hkv, vd=vd, talk=self.talk, gates=gates)
-            o = mixed
-        self.out.forward(o, accumulate_into=residual, next_norm=next_norm)
+            heads = self.rt.empty(T, H * vd)
+            ops.head_mix_gate(o, heads, H=H, Hkv=Hkv, vd=vd, talk=self.talk, gates=gates)
+        self.out.forward(heads, accumulate_into=residual, next_norm=next_norm)
