@@ -153,9 +153,10 @@ def conv_rotary_attention(n, W, m, eps, rnd=_same):
     T = n.shape[0]
     H, G, dk, dv, scale = m["heads"], m["kv_heads"], m["dim"], m["vdim"], m["scale"]
     pos = torch.arange(T)
-    q = rnd(short_convolution(rnd(n @ W["q"].T), W["q.conv"])).view(T, H, dk)
-    k = rnd(short_convolution(rnd(n @ W["k"].T), W["k.conv"])).view(T, G, dk)
-    v = rnd(short_convolution(rnd(n @ W["v"].T), W["v.conv"])).view(T, G, dv)
+    conv = lambda u, name: rnd(short_convolution(u, W[name])) if name in W else u          # (no taps: as projected)
+    q = conv(rnd(n @ W["q"].T), "q.conv").view(T, H, dk)
+    k = conv(rnd(n @ W["k"].T), "k.conv").view(T, G, dk)
+    v = conv(rnd(n @ W["v"].T), "v.conv").view(T, G, dv)
     q, k = plain_norm(q, W["q.norm"], eps), plain_norm(k, W["k.norm"], eps)
     rot = m.get("rot")
     if rot and rot.get("dims"):
