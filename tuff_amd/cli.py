@@ -73,6 +73,12 @@ def build_parser() -> argparse.ArgumentParser:
     return ap
 
 
+def _part_name(part) -> str:
+    """A part's class; one made of two side by side names them too."""
+    inner = [getattr(part, side) for side in ("left", "right") if hasattr(part, side)]
+    return type(part).__name__ + (f"({' | '.join(_part_name(p) for p in inner)})" if inner else "")
+
+
 def _inspect(cfg, model, out=sys.stdout) -> None:
     """Inventory in the spirit of lfm25_model_print_inspection (src/lfm25_model.c:381-401)."""
     print(f"architecture: {cfg.architecture}", file=out)
@@ -84,7 +90,7 @@ def _inspect(cfg, model, out=sys.stdout) -> None:
     for i, b in enumerate(model.blocks):
         # a block of another arrangement may have neither a mixer nor a feed-forward of these names
         mixer, ffn = getattr(b, "mixer", None), getattr(b, "ffn", None)
-        inside = " + ".join(type(p).__name__ for p in (mixer, ffn) if p is not None) or type(b).__name__
+        inside = " + ".join(_part_name(p) for p in (mixer, ffn) if p is not None) or type(b).__name__
         spec = mixer.cache_spec() if hasattr(mixer, "cache_spec") else None
         print(f"  layer {i}: {type(b).__name__}: {inside}  cache: {spec}", file=out)
     print(f"run order: {[r.block for r in model.schedule]}", file=out)
