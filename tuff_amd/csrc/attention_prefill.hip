@@ -22,6 +22,15 @@
 //
 // Cache layout: K [page][kv_head][offset][hd], V [page][kv_head][hd][offset]; page size a
 // multiple of 16, head size a multiple of 8.
+//
+// The wide form of the kernel (EX) adds: values of another width than the keys (V [page][kv_head][vd][offset];
+// the tiles are as wide as the wider of the two and the narrower one's missing channels are zeros); a
+// logarithmic distance penalty r1_h * ln(1 + r2_h * (position - key)) off the scaled score; weights that keep
+// float32's precision through the matrix cores (a weight p goes in as two bfloat16 numbers, p rounded and
+// what the rounding left, in two products); and every query head's weights applied to the values of every kv
+// head (all_v: the grid's second axis is the kv head whose values are read, the sums are written in float32
+// as [token][head][kv head][vd]), from which a following kernel forms heads whose weights are mixtures of
+// the heads' softmax weights.
 #include "common.h"
 #include <math.h>
 
@@ -42,14 +51,22 @@ __device__ __forceinline__ int k_row_of_key(int key) {
     return sub * 32 + kb * 16 + h * 8 + q * 4 + m;
 }
 
-template <int HDP, int NBW, int AHEAD>
+struct WideArgs {
+    int vd;                     // channels of a value
+    const float* log_r1;        // [H] or null
+    const float* log_r2;        // [H]
+    int all_v;
+    float* out_wide;            // all_v: float32 [token][head][kv head][vd]
+};
+
+template <int HDP, int NBW, int AHEAD, bool EX>
 __global__ __launch_bounds__(NT) void attn_prefill_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
     bf16_t* __restrict__ out, const int* __restrict__ block_table, int max_blocks,
     const int2* __restrict__ blk, const int4* __restrict__ req_info,
     int H, int Hkv, int hd, int page_size, int window, float scale_log2e,
     int seg_keys, float* __restrict__ ws_o, float* __restrict__ ws_ml, const float* __restrict__ sinks,
-    const float* __restrict__ slopes) {
+    const float* __restrict__ slopes, WideArgs wide) {
     constexpr int KC = HDP / 32;          // 32-wide chunks of the head dimension
     constexpr int DB = HDP / 16;          // 16-wide blocks of output channels
     constexpr int HC = HDP / 8;           // 16-byte chunks of a K row
@@ -69,6 +86,9 @@ __global__ __launch_bounds__(NT) void attn_prefill_kernel(
     const int qb = blockIdx.x / Hkv;
     const int kvh = blockIdx.x % Hkv;
     const int G = H / Hkv;
+    const int vd = EX ? wide.vd : hd;
+    const int vh = (EX && wide.all_v) ? (int)blockIdx.y : kvh;          // the kv head whose values are read
+    const bool log_dist = EX && wide.log_r1 != nullptr;
     int r = qb, col0 = 0;
     if (blk) { const int2 b = blk[qb]; r = b.x; col0 = b.y; }
     const int4 info = req_info[r];         // (first token of the request in the step, tokens, first position, -)
@@ -91,6 +111,7 @@ __global__ __launch_bounds__(NT) void attn_prefill_kernel(
     const int wcol0 = col0 + wave * NBW * 16;
     int pos_c[NBW], lo_c[NBW];
     float slope_c[NBW];                    // the head's distance slope, in base-2 exponents; 0: none
+    float r1_c[NBW], r2_c[NBW];            // the head's logarithmic penalty: r1 * log2(1 + r2 * distance) in base-2 exponents
     long long qrow[NBW];                   // row of the column in q and out; -1: no column
     bf16x8 qf[NBW][KC];
     int wave_pos_max = -1, wave_pos_min = 0x7fffffff, wave_lo_max = 0;
@@ -101,6 +122,8 @@ __global__ __launch_bounds__(NT) void attn_prefill_kernel(
         const int tok = t0 + (valid ? c / G : 0);
         const int head = kvh * G + (valid ? c % G : 0);
         slope_c[nb] = slopes ? slopes[head] * 1.4426950408889634f : 0.f;
+        r1_c[nb] = log_dist ? wide.log_r1[head] : 0.f;
+        r2_c[nb] = log_dist ? wide.log_r2[head] : 0.f;
         pos_c[nb] = valid ? pos0 + c / G : -1;
         lo_c[nb] = (valid && window > 0) ? max(0, pos_c[nb] - window + 1) : 0;
         qrow[nb] = valid ? (long long)tok * H + head : -1;
@@ -181,19 +204,21 @@ __global__ __launch_bounds__(NT) void attn_prefill_kernel(
         v_gran[i] = __builtin_amdgcn_readfirstlane(c8 / 2);
         v_key[i] = c8 * 8;
         v_off[i] = dim * page_size + (c8 % 2) * 8;
-        v_ok[i] = dim < hd;
+        v_ok[i] = dim < vd;
         v_lds[i] = dim * VROW + c8 * 8;
     }
-    const bool whole_rows = hd == HDP;
-    const unsigned page_stride = (unsigned)(Hkv * page_size * hd);       // elements of a page in either cache (the host checks that it fits)
+    const bool whole_rows = hd == HDP && vd == HDP;
+    const unsigned page_stride = (unsigned)(Hkv * page_size * hd);       // elements of a page in the key cache (the host checks that it fits)
     const unsigned head_off = (unsigned)(kvh * page_size * hd);          // this kv head's share of it
+    const unsigned page_stride_v = (unsigned)(Hkv * page_size * vd);     // the same of the value cache
+    const unsigned head_off_v = (unsigned)(vh * page_size * vd);
     const int ps_mask = (page_size & (page_size - 1)) == 0 ? page_size - 1 : 0;   // a power of two: offsets wrap by a mask
     int ld_off = key_start % page_size;                 // offset in its page of the first key of the next step to load
     auto load_step = [&](int set, int s, int pages) {   // step s of the block -> register set; zeros beyond pos_max
         const int key0 = key_start + s * STEP;
         const int gslot0 = (s % 16) * 4;                // granule of the step's first key within `pages`
         // per piece, the same for the lanes of a wave: where its granule's rows start (-1: no such page)
-        auto granule = [&](int g4, long long& base, int& go) {
+        auto granule = [&](int g4, long long& base, int& go, bool values) {
             const int page = __builtin_amdgcn_readlane(pages, gslot0 + g4);
             go = ld_off + 16 * g4;
             if (ps_mask) go &= ps_mask;
@@ -202,21 +227,22 @@ __global__ __launch_bounds__(NT) void attn_prefill_kernel(
                 for (int w = 0; w < 3; ++w)
                     if (go >= page_size) go -= page_size;
             }
-            base = page >= 0 ? (long long)((unsigned long long)(unsigned)page * page_stride + head_off) : -1;
+            if (EX && values) base = page >= 0 ? (long long)((unsigned long long)(unsigned)page * page_stride_v + head_off_v) : -1;
+            else base = page >= 0 ? (long long)((unsigned long long)(unsigned)page * page_stride + head_off) : -1;
         };
         long long bk[KPT], bv[VPT];
         bool all_live = key0 + STEP - 1 <= pos_max;
 #pragma unroll
         for (int i = 0; i < KPT; ++i) {
             int go;
-            granule(k_gran[i], bk[i], go);
+            granule(k_gran[i], bk[i], go, false);
             all_live = all_live && bk[i] >= 0;
             bk[i] += (long long)go * hd;                // (-1 stays negative: go * hd < page_stride)
         }
 #pragma unroll
         for (int i = 0; i < VPT; ++i) {
             int go;
-            granule(v_gran[i], bv[i], go);
+            granule(v_gran[i], bv[i], go, true);
             all_live = all_live && bv[i] >= 0;
             bv[i] += go;
         }
@@ -293,6 +319,7 @@ __global__ __launch_bounds__(NT) void attn_prefill_kernel(
         if (open || live0) sc[0] = scores(buf, 0);
         if (open || live1) sc[1] = scores(buf, 1);
         bf16x8 pf[2][NBW];
+        bf16x8 pf_lo[EX ? 2 : 1][NBW];       // what rounding a weight to bfloat16 left
         float corr[NBW];
         bool same = true;
 #pragma unroll
@@ -302,7 +329,7 @@ __global__ __launch_bounds__(NT) void attn_prefill_kernel(
             // it is the same instruction with and without the mask.
             float mx = -INFINITY;
             bool ok[2][8];
-            if (slopes) {
+            if (slopes || log_dist) {
                 // Heads with a distance slope: slope * (position - key) is taken off the scaled score (from the
                 // integer distance, so that far positions lose no bits).  The scores become exponents here, the
                 // maximum is theirs, and the scale below is 1.
@@ -313,10 +340,13 @@ __global__ __launch_bounds__(NT) void attn_prefill_kernel(
 #pragma unroll
                         for (int e = 0; e < 4; ++e) {
                             const int key = key0 + 32 * sub + 8 * g + 4 * kb + e;
-                            sc[sub].v[kb][nb][e] = fmaf(sc[sub].v[kb][nb][e], scale_log2e, slope_c[nb] * (float)(key - pos_c[nb]));
+                            float z = fmaf(sc[sub].v[kb][nb][e], scale_log2e, slope_c[nb] * (float)(key - pos_c[nb]));
+                            // (ln(1 + x) log2(e) = log2(1 + x); keys after the position are masked below)
+                            if (log_dist) z -= r1_c[nb] * __builtin_amdgcn_logf(fmaf(r2_c[nb], (float)max(pos_c[nb] - key, 0), 1.0f));
+                            sc[sub].v[kb][nb][e] = z;
                         }
             }
-            const float unit = slopes ? 1.f : scale_log2e;
+            const float unit = (slopes || log_dist) ? 1.f : scale_log2e;
 #pragma unroll
             for (int sub = 0; sub < 2; ++sub)
 #pragma unroll
@@ -344,6 +374,7 @@ __global__ __launch_bounds__(NT) void attn_prefill_kernel(
                 for (int i = 0; i < 8; ++i) {
                     const float p = ok[sub][i] ? __builtin_amdgcn_exp2f(fmaf(sc[sub].v[i / 4][nb][i % 4], unit, -m_safe)) : 0.f;
                     pf[sub][nb][i] = (bf16_t)p;
+                    if (EX) pf_lo[EX ? sub : 0][nb][i] = (bf16_t)(p - (float)pf[sub][nb][i]);
                 }
             m_run[nb] = m_new;
         }
@@ -365,10 +396,16 @@ __global__ __launch_bounds__(NT) void attn_prefill_kernel(
             for (int db = 0; db < DB; ++db) {
                 const bf16x8 vf = *(const bf16x8*)(Vb + db * 16 * VROW + sub * 32);
 #pragma unroll
-                for (int nb = 0; nb < NBW; ++nb) o[db][nb] = mfma32(vf, pf[sub][nb], o[db][nb]);
+                for (int nb = 0; nb < NBW; ++nb) {
+                    o[db][nb] = mfma32(vf, pf[sub][nb], o[db][nb]);
+                    if (EX) o[db][nb] = mfma32(vf, pf_lo[EX ? sub : 0][nb], o[db][nb]);
+                }
             }
 #pragma unroll
-            for (int nb = 0; nb < NBW; ++nb) l_acc[nb] = mfma32(ones, pf[sub][nb], l_acc[nb]);
+            for (int nb = 0; nb < NBW; ++nb) {
+                l_acc[nb] = mfma32(ones, pf[sub][nb], l_acc[nb]);
+                if (EX) l_acc[nb] = mfma32(ones, pf_lo[EX ? sub : 0][nb], l_acc[nb]);
+            }
         }
     };
 
@@ -423,24 +460,36 @@ __global__ __launch_bounds__(NT) void attn_prefill_kernel(
             const float keep = __builtin_amdgcn_exp2f(m_run[nb] - m_all);
             inv = keep / (l * keep + __builtin_amdgcn_exp2f(s2 - m_all));
         }
+        if (EX && wide.all_v) {
+            float* dst = wide.out_wide + (qrow[nb] * Hkv + vh) * vd;
+#pragma unroll
+            for (int db = 0; db < DB; ++db) {
+                const int dim = db * 16 + 4 * g;
+                if (dim < vd) {
+                    const f32x4 v = o[db][nb];
+                    *(f32x4*)(dst + dim) = f32x4{v[0] * inv, v[1] * inv, v[2] * inv, v[3] * inv};
+                }
+            }
+            continue;
+        }
 #pragma unroll
         for (int db = 0; db < DB; ++db) {
             const int dim = db * 16 + 4 * g;
-            if (dim < hd) {
+            if (dim < vd) {
                 const f32x4 v = o[db][nb];
                 bf16x4 w = {(bf16_t)(v[0] * inv), (bf16_t)(v[1] * inv), (bf16_t)(v[2] * inv), (bf16_t)(v[3] * inv)};
-                *(bf16x4*)(out + qrow[nb] * hd + dim) = w;
+                *(bf16x4*)(out + qrow[nb] * vd + dim) = w;
             }
         }
     }
 }
 
-template <int HDP, int NBW, int AHEAD>
+template <int HDP, int NBW, int AHEAD, bool EX = false>
 int launch(dim3 grid, hipStream_t stream, const bf16_t* q, const bf16_t* kc, const bf16_t* vc, bf16_t* out,
            const int* bt, int max_blocks, const int2* blk, const int4* req_info,
            int H, int Hkv, int hd, int ps, int window, float scale_log2e, int seg_keys, float* ws_o, float* ws_ml,
-           const float* sinks, const float* slopes) {
-    auto kern = attn_prefill_kernel<HDP, NBW, AHEAD>;
+           const float* sinks, const float* slopes, WideArgs wide = WideArgs{0, nullptr, nullptr, 0, nullptr}) {
+    auto kern = attn_prefill_kernel<HDP, NBW, AHEAD, EX>;
     constexpr int lds = 2 * (STEP * (HDP + 8) + HDP * VROW) * 2;
     static bool set = false;
     if (!set) {
@@ -448,7 +497,7 @@ int launch(dim3 grid, hipStream_t stream, const bf16_t* q, const bf16_t* kc, con
         set = true;
     }
     hipLaunchKernelGGL(kern, grid, dim3(NT), lds, stream, q, kc, vc, out, bt, max_blocks, blk, req_info,
-                       H, Hkv, hd, ps, window, scale_log2e, seg_keys, ws_o, ws_ml, sinks, slopes);
+                       H, Hkv, hd, ps, window, scale_log2e, seg_keys, ws_o, ws_ml, sinks, slopes, wide);
     return launch_status();
 }
 }  // namespace
@@ -510,4 +559,32 @@ TUFF_EXPORT int tuff_attention_prefill(const void* q, const void* k_cache, const
                                        hipStream_t stream) {
     return tuff_attention_prefill_sinks(q, k_cache, v_cache, out, block_table, max_blocks, blk, n_qblocks, req_info, H, Hkv, hd,
                                         page_size, window, scale, n_segs, seg_keys, ws_o, ws_ml, nullptr, stream);
+}
+
+// The wide form: values vd channels wide (V [page][kv_head][vd][offset]), weights that keep float32's precision,
+// log_r1, log_r2 (float32 [H], or both null): r1[h] * ln(1 + r2[h] * (position - key)) is taken off head h's scaled
+// scores.  all_v: every head's weights on every kv head's values, out is then float32 [tokens][H][Hkv][vd]; else out
+// is bfloat16 [tokens][H][vd].  Keys are not cut into segments.
+TUFF_EXPORT int tuff_attention_prefill_wide(const void* q, const void* k_cache, const void* v_cache, void* out,
+                                            const int* block_table, int max_blocks, const int* blk, int n_qblocks,
+                                            const int* req_info, int H, int Hkv, int hd, int vd, int page_size, int window,
+                                            float scale, const float* sinks, const float* slopes, const float* log_r1,
+                                            const float* log_r2, int all_v, hipStream_t stream) {
+    if (n_qblocks <= 0) return 0;
+    if (hd > 256 || hd % 8 != 0 || vd > 256 || vd <= 0 || vd % 8 != 0 || page_size % 16 != 0 || Hkv <= 0 || H % Hkv != 0) return -2;
+    if (Hkv > 65535 || !(scale > 0.f) || (log_r1 == nullptr) != (log_r2 == nullptr)) return -2;
+    if ((long long)Hkv * page_size * max(hd, vd) > 0x7fffffffll || (long long)n_qblocks * Hkv > 0x7fffffffll) return -2;
+    dim3 grid(n_qblocks * Hkv, all_v ? Hkv : 1, 1);
+    const float sl = scale * 1.4426950408889634f;
+    const WideArgs wide{vd, log_r1, log_r2, all_v, all_v ? (float*)out : nullptr};
+    const int widest = max(hd, vd);
+#define GO(HDP, NBW, AHEAD) return launch<HDP, NBW, AHEAD, true>(grid, stream, (const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache, \
+        (bf16_t*)out, block_table, max_blocks, (const int2*)blk, (const int4*)req_info, H, Hkv, hd, page_size, window, sl, 0, nullptr, \
+        nullptr, sinks, slopes, wide)
+    if (widest <= 32) GO(32, 2, 3);
+    else if (widest <= 64) GO(64, 2, 2);
+    else if (widest <= 96) GO(96, 2, 2);
+    else if (widest <= 128) GO(128, 2, 2);
+    else GO(256, 2, 1);
+#undef GO
 }

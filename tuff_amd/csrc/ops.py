@@ -152,6 +152,9 @@ _SIGNATURES = {
         "tuff_attention_prefill_biased": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_void_p, _c_int,
                                           _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_int,
                                           _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p],
+        "tuff_attention_prefill_wide": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_void_p, _c_int,
+                                        _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float,
+                                        _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_void_p],
         "tuff_attention_prefill_block_columns": [_c_int],
     },
     "shortconv": {
@@ -1247,6 +1250,62 @@ def attention_prefill(q, k_cache, v_cache, out, *, block_table, blocks, req_info
         _check(load("attention_prefill").tuff_attention_prefill_sinks(*args, sinks.data_ptr(), _stream()), "attention_prefill")
         if merge is not None:
             _check(load("attention_mfma").tuff_attention_merge_sinks(*merge, sinks.data_ptr(), _stream()), "attention_merge")
+
+
+def attention_prefill_wide_supported(dtype, hd: int, vd: int, page_size: int) -> bool:
+    return dtype == torch.bfloat16 and hd % 8 == 0 and vd % 8 == 0 and max(hd, vd) <= 256 and page_size % 16 == 0
+
+
+def attention_prefill_wide(q, k_cache, v_cache, out, *, block_table, blocks, req_info, H, Hkv, hd, vd, page_size, max_ctx_len,
+                           window=0, scale=None, sinks=None, slopes=None, log_distance=None, all_values: bool = False) -> None:
+    """attention_prefill's kernel in its wide form: values of vd channels (v_cache [P, Hkv, vd, page_size]), softmax
+    weights that keep float32's precision through the matrix cores, and optionally log_distance = (r1, r2), float32 [H]
+    each: r1[h] * ln(1 + r2[h] * (position - key)) is taken off head h's scaled scores.  all_values: every query head's
+    weights are applied to the values of every kv head and out is float32 [T, H * Hkv * vd] (head, kv head, channel), for
+    head_mix_gate; otherwise out is bfloat16 [T, H * vd].  The keys are not cut into segments."""
+    T = q.shape[0]
+    if not attention_prefill_wide_supported(q.dtype, hd, vd, page_size):
+        raise KernelError(f"attention_prefill_wide: needs bfloat16, head sizes that are multiples of 8 (got {hd}, {vd}) "
+                          f"and a page size that is a multiple of 16 (got {page_size})")
+    _opt("sinks", sinks, torch.float32, (H,))
+    _opt("slopes", slopes, torch.float32, (H,))
+    r1 = r2 = None
+    if log_distance is not None:
+        r1, r2 = log_distance
+        _gpu("log_distance r1", r1, torch.float32, (H,))
+        _gpu("log_distance r2", r2, torch.float32, (H,))
+    _gpu("q", q, torch.bfloat16, (T, H * hd))
+    if all_values:
+        _gpu("out", out, torch.float32, (T, H * Hkv * vd))
+    else:
+        _gpu("out", out, torch.bfloat16, (T, H * vd))
+    P = k_cache.shape[0]
+    _gpu("k_cache", k_cache, torch.bfloat16, (P, Hkv, page_size, hd))
+    _gpu("v_cache", v_cache, torch.bfloat16, (P, Hkv, vd, page_size))
+    _gpu("block_table", block_table, torch.int32)
+    R = req_info.shape[0]
+    _gpu("req_info", req_info, torch.int32, (R, 4))
+    if block_table.dim() != 2 or block_table.shape[0] != R:
+        raise KernelError("attention_prefill_wide: block_table must be [requests, blocks]")
+    if block_table.shape[1] * page_size < int(max_ctx_len):
+        raise KernelError("attention_prefill_wide: block_table is narrower than the longest context")
+    if H % Hkv:
+        raise KernelError("attention_prefill_wide: the query heads must be a multiple of the kv heads")
+    if blocks is None:
+        if H // Hkv > attention_prefill_block_columns(max(hd, vd)):
+            raise KernelError("attention_prefill_wide: without a block list a request's columns must fit one block")
+        nblk = R
+    else:
+        nblk = blocks.shape[0]
+        _gpu("blocks", blocks, torch.int32, (nblk, 2))
+    if scale is None:
+        scale = 1.0 / math.sqrt(hd)
+    _check(load("attention_prefill").tuff_attention_prefill_wide(
+        q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), out.data_ptr(), block_table.data_ptr(), block_table.shape[1],
+        None if blocks is None else blocks.data_ptr(), nblk, req_info.data_ptr(), H, Hkv, hd, vd, page_size, int(window or 0),
+        float(scale), None if sinks is None else sinks.data_ptr(), None if slopes is None else slopes.data_ptr(),
+        None if r1 is None else r1.data_ptr(), None if r2 is None else r2.data_ptr(), int(bool(all_values)), _stream()),
+        "attention_prefill_wide")
 
 
 def query_blocks(q_len, G: int, nb: int, ctx_len=None):

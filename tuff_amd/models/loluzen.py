@@ -42,7 +42,7 @@ def _mixer(cfg: LoluzenConfig, i: int):
     if layer["type"] == "parallel":
         a, r = m["left"], m["right"]
         lp, rp = p + "left.", p + "right."
-        left = AttentionMixer(d, a["heads"], a["kv_heads"], a["dim"], value_dim=a["vdim"], scale=a["scale"],
+        left = AttentionMixer(d, a["heads"], a["kv_heads"], a["dim"], value_dim=a["vdim"], scale=a["scale"], exact_weights=True,
                               names={k: lp + k for k in ("q", "k", "v", "o", "q.b", "k.b", "v.b", "r1", "r2", "talk", "g")})
         right = ForgetGateMixer(d, r["heads"], r["dim"], r["vdim"], cfg.eps,
                                 names={k: rp + k for k in ("q", "f", "f.b", "lower", "v", "norm", "o")})
@@ -59,7 +59,7 @@ def _mixer(cfg: LoluzenConfig, i: int):
         for k in ("q.conv", "k.conv", "v.conv"):
             names.pop(k)
     return AttentionMixer(d, m["heads"], m["kv_heads"], m["dim"], value_dim=m["vdim"], scale=m["scale"],
-                          qk_norm_eps=cfg.eps, position=position, conv_taps=taps, names=names)
+                          qk_norm_eps=cfg.eps, position=position, conv_taps=taps, names=names, exact_weights=True)
 
 
 def _feed_forward(cfg: LoluzenConfig, i: int):

@@ -77,7 +77,19 @@ class PagedAttention:
     def attend(self, q, o, ctx, cache, g) -> None:
         G = self.H // self.Hkv
         log_distance, talk = getattr(self, "log_distance", None), getattr(self, "talk", None)
-        if log_distance is not None or talk is not None:
+        exact = getattr(self, "exact_weights", False)
+        if ((log_distance is not None or talk is not None or exact) and ctx.max_q_len > 1
+                and ops.attention_prefill_wide_supported(q.dtype, self.hd, self.vd, cache.page_size)):
+            # prompt portions in the step: the matrix-core kernel in its wide form (single tokens beside them are blocks
+            # of one token's heads)
+            nb = ops.attention_prefill_block_columns(max(self.hd, self.vd)) // 16
+            ops.attention_prefill_wide(q, cache.k, cache.v, o, block_table=g.block_table,
+                                       blocks=self._blocks(ctx, G, nb, q.device, longest_first=True), req_info=ctx.req_info,
+                                       H=self.H, Hkv=self.Hkv, hd=self.hd, vd=self.vd, page_size=cache.page_size,
+                                       max_ctx_len=ctx.max_ctx_len, window=self.window or 0, scale=self.scale, sinks=self.sinks,
+                                       slopes=self.slopes, log_distance=log_distance, all_values=talk is not None)
+            return
+        if log_distance is not None or talk is not None or exact:
             ops.attention_general(q, cache.k, cache.v, o, block_table=g.block_table,
                                   req_of_token=ctx.req_of_token, positions=ctx.positions,
                                   H=self.H, Hkv=self.Hkv, hd=self.hd, page_size=cache.page_size,
@@ -123,7 +135,8 @@ class AttentionMixer(Mixer, PagedAttention):
                  names: dict[str, str], qk_norm_eps: Optional[float] = None,
                  position: Optional[PositionEncoding] = None, window: Optional[int] = None,
                  scale: Optional[float] = None, aliases: Optional[dict[str, tuple]] = None,
-                 value_dim: Optional[int] = None, slope_span: Optional[float] = None, conv_taps: Optional[int] = None):
+                 value_dim: Optional[int] = None, slope_span: Optional[float] = None, conv_taps: Optional[int] = None,
+                 exact_weights: bool = False):
         """names: checkpoint names of 'q', 'k', 'v', 'o' and, with qk_norm_eps, 'q_norm', 'k_norm' (without these
         two names the norm has no weight: q and k are divided by their root mean square over the head); with a
         'sink' among them the heads have sinks.  value_dim: width of a value head (default: head_dim).
@@ -131,7 +144,10 @@ class AttentionMixer(Mixer, PagedAttention):
         Further names switch further options on: 'q.b', 'k.b', 'v.b' biases of the projections; 'r1', 'r2' [H] the
         logarithmic distance penalty; 'talk' [H, H] the matrix that mixes the heads' softmax weights; 'g' [H, d] the
         gate per head; with conv_taps, 'q.conv', 'k.conv', 'v.conv' [channels, taps] the convolutions' taps (one tap: a
-        factor per channel and no state)."""
+        factor per channel and no state).
+        exact_weights: the softmax weights keep float32's precision where they meet the values, also with bfloat16
+        activations (the kernels that round them to bfloat16 for the matrix cores are not used)."""
+        self.exact_weights = bool(exact_weights)
         if num_heads % num_kv_heads:
             raise ValueError(f"heads {num_heads} must be a multiple of kv heads {num_kv_heads}")
         if head_dim > 256:
@@ -267,6 +283,7 @@ class AttentionMixer(Mixer, PagedAttention):
         k = None if fused else self.rt.empty(T, Hkv * hd)
 
         one_kernel = (fused and tables is not None and ctx.max_q_len == 1 and self.sinks is None and self.talk is None
+                      and not self.exact_weights
                       and self.log_distance is None and ops.attention_decode_fused_supported(
             qkv.dtype, H, Hkv, hd, cache.page_size, tables[1], tables[2]))
 
