@@ -244,6 +244,92 @@ def test_attention_with_mixed_heads_one_key_stands_out(gpu, dk, dv, H, G, dtype)
                 assert err <= tol * max(1.0, float(want.abs().max())), (n, special, i, float(err))
 
 
+def _paged_case(gpu, H, Hkv, hd, vd, reqs, opts, ps=16, seed=0):
+    """Scattered pages of random bfloat16 keys and values for requests (tokens before the step, tokens of the step), queries,
+    and the options' tensors; everything a kernel's launch takes."""
+    gen = torch.Generator().manual_seed(seed)
+    rnd = lambda *shape: torch.randn(*shape, generator=gen)
+    R, T = len(reqs), sum(n for _, n in reqs)
+    longest = max(c + n for c, n in reqs)
+    nblk = -(-longest // ps)
+    P = R * nblk + 3
+    table = torch.randperm(P, generator=gen)[:R * nblk].view(R, nblk).int().to(gpu)
+    i32 = lambda a: torch.tensor(a, dtype=torch.int32, device=gpu)
+    req_of, pos, info, t = [], [], [], 0
+    for r, (c, n) in enumerate(reqs):
+        info.append((t, n, c, 0)); req_of += [r] * n; pos += list(range(c, c + n)); t += n
+    window, sinks, slopes, logd, talk, gate = opts
+    case = dict(q=(rnd(T, H * hd) * 1.5).bfloat16().to(gpu), k=rnd(P, Hkv, ps, hd).bfloat16().to(gpu), v=rnd(P, Hkv, vd, ps).bfloat16().to(gpu),
+                table=table, req_of=i32(req_of), pos=i32(pos), info=i32(info), longest=longest, T=T, window=window,
+                sinks=(rnd(H) + 1).to(gpu) if sinks else None, slopes=(torch.rand(H, generator=gen) * 0.1).to(gpu) if slopes else None,
+                logd=((torch.rand(H, generator=gen) + 0.2).to(gpu), (torch.rand(H, generator=gen) * 2 + 0.1).to(gpu)) if logd else None,
+                talk=rnd(H, H).to(gpu) if talk else None, gates=rnd(T, H).to(gpu) if gate else None)
+    return case
+
+
+def _general(c, H, Hkv, hd, vd, ps=16):
+    """The one-wave-a-head kernel (float32 weights; held to the plain functions by the float32 tests above), then the
+    heads' mixing and gates: [T, H * vd] float32."""
+    from tuff_amd.csrc import ops
+    mixed = c["talk"] is not None
+    o = torch.zeros((c["T"], H * Hkv * vd) if mixed else (c["T"], H * vd), dtype=torch.float32 if mixed else torch.bfloat16, device=c["q"].device)
+    ops.attention_general(c["q"], c["k"], c["v"], o, block_table=c["table"], req_of_token=c["req_of"], positions=c["pos"], H=H, Hkv=Hkv,
+                          hd=hd, page_size=ps, window=c["window"], scale=0.2, vd=vd, sinks=c["sinks"], slopes=c["slopes"],
+                          log_distance=c["logd"], all_values=mixed)
+    if not mixed and c["gates"] is None:
+        return o.float()
+    out = torch.zeros(c["T"], H * vd, dtype=o.dtype, device=o.device)
+    ops.head_mix_gate(o, out, H=H, Hkv=Hkv, vd=vd, talk=c["talk"], gates=c["gates"])
+    return out.float()
+
+
+SHAPES = [(4, 2, 64, 64), (4, 4, 96, 64), (6, 3, 24, 40), (2, 1, 128, 128), (8, 2, 40, 16), (2, 2, 256, 64), (40, 2, 16, 8), (3, 3, 8, 256)]
+# (window, sinks, slopes, logarithmic penalty, mixed heads, gates)
+OPTIONS = [(0, 0, 0, 0, 0, 0), (48, 0, 0, 0, 0, 0), (0, 1, 0, 0, 0, 1), (300, 1, 0, 0, 0, 0), (0, 0, 1, 0, 0, 0), (0, 0, 0, 1, 0, 0),
+           (0, 0, 0, 1, 1, 1), (100, 1, 0, 1, 1, 0)]
+
+
+@pytest.mark.parametrize("H, Hkv, hd, vd", SHAPES)
+def test_prompt_kernel_in_its_wide_form_against_the_general_kernel(gpu, H, Hkv, hd, vd):
+    """Portions at the start, far into a request and across page and step borders, a single token among them; float32
+    sums where the heads are mixed agree to float32's rounding: the weights keep their precision through the matrix cores."""
+    from tuff_amd.csrc import ops
+    reqs = [(0, 70), (130, 5), (300, 1), (17, 200)]
+    for opts in OPTIONS:
+        c = _paged_case(gpu, H, Hkv, hd, vd, reqs, opts, seed=H + hd)
+        c["gates"] = None
+        want = _general(c, H, Hkv, hd, vd)
+        mixed = c["talk"] is not None
+        o = torch.zeros((c["T"], H * Hkv * vd) if mixed else (c["T"], H * vd), dtype=torch.float32 if mixed else torch.bfloat16, device=gpu)
+        blocks = torch.from_numpy(ops.query_blocks(np.array([n for _, n in reqs]), H // Hkv, 8, np.array([a + n for a, n in reqs]))).to(gpu)
+        ops.attention_prefill_wide(c["q"], c["k"], c["v"], o, block_table=c["table"], blocks=blocks, req_info=c["info"], H=H, Hkv=Hkv, hd=hd,
+                                   vd=vd, page_size=16, max_ctx_len=c["longest"], window=c["window"], scale=0.2, sinks=c["sinks"],
+                                   slopes=c["slopes"], log_distance=c["logd"], all_values=mixed)
+        if mixed:
+            got = torch.zeros(c["T"], H * vd, dtype=torch.float32, device=gpu)
+            ops.head_mix_gate(o, got, H=H, Hkv=Hkv, vd=vd, talk=c["talk"], gates=None)
+        else:
+            got = o.float()
+        tol = 3e-5 if mixed else 0.01
+        assert (got - want).abs().max() <= tol * max(1.0, float(want.abs().max())), opts
+
+
+@pytest.mark.parametrize("H, Hkv, hd, vd", SHAPES)
+def test_single_token_kernels_with_float32_weights_against_the_general_kernel(gpu, H, Hkv, hd, vd):
+    """Single tokens at the first position, on both sides of a part's 256 keys and far behind them."""
+    from tuff_amd.csrc import ops
+    reqs = [(n, 1) for n in (0, 5, 255, 256, 257, 700, 1023, 15)]
+    for opts in OPTIONS:
+        c = _paged_case(gpu, H, Hkv, hd, vd, reqs, opts, seed=H + vd)
+        want = _general(c, H, Hkv, hd, vd)
+        got = torch.zeros(c["T"], H * vd, dtype=torch.float32, device=gpu)
+        ops.attention_decode_exact(c["q"], c["k"], c["v"], got, block_table=c["table"], req_of_token=c["req_of"], positions=c["pos"], H=H,
+                                   Hkv=Hkv, hd=hd, vd=vd, page_size=16, max_ctx_len=c["longest"], window=c["window"], scale=0.2,
+                                   sinks=c["sinks"], slopes=c["slopes"], log_distance=c["logd"], talk=c["talk"], gates=c["gates"])
+        tol = 3e-5 if c["talk"] is not None else 0.01            # (the general kernel's own output is bfloat16 where heads are not mixed)
+        assert (got - want).abs().max() <= tol * max(1.0, float(want.abs().max())), opts
+
+
 def test_forget_scan_carries_its_state_across_any_cut(gpu):
     """The recurrence's kernel on its own, at key sizes on both sides of a wave's 64 lanes and value sizes of one and
     several blocks: a sequence in one call against the same sequence in portions of 1, 2 and more through the state, in

@@ -188,3 +188,264 @@ TUFF_EXPORT int tuff_head_mix_gate(const void* o, int in_dt, const float* talk, 
 #undef LAUNCH
     return launch_status();
 }
+
+// ---------------------------------------------------------------------------------------------------------------
+// Single tokens over a bfloat16 cache with float32 weights, in three kernels, so that the keys and the values of a
+// request are read once whatever the number of query heads:
+//   scores   a workgroup a (token, kv head, part of 256 keys), a thread a key: the key's row is read in 16-byte
+//            pieces and meets the queries of all heads of the group (from LDS); the scaled scores, penalties taken
+//            off, go to S [token][head][key] and the part's maximum and sum of exponentials per head to ml.
+//   values   a workgroup a (token, kv head, part): from ml every head's maximum and sum over all parts (with its
+//            sink); a thread a key forms the key's normalised weight for every head of the group, or, with a mixing
+//            matrix, sum_g talk[h][g] w_g from the weights of all heads; then the threads, each a value channel and
+//            a share of the part's pages, sum weight * value for the group's heads; partial sums per part go to po.
+//   merge    out[token][head] = gate * sum over the parts that hold a visible key.
+// Heads are taken sixteen at a time.  Layouts as above: K [page][kv head][offset][hd], V [page][kv head][vd][offset].
+namespace {
+constexpr int DEC_KEYS = 256;         // keys a part, threads a workgroup
+constexpr int DEC_HEADS = 16;         // heads of a group taken together
+constexpr int DEC_MAX_H = 256;
+
+__device__ __forceinline__ float block_max_256(float v, float* scratch) {
+    v = wave_max(v);
+    __syncthreads();
+    if (threadIdx.x % WAVE == 0) scratch[threadIdx.x / WAVE] = v;
+    __syncthreads();
+    return fmaxf(fmaxf(scratch[0], scratch[1]), fmaxf(scratch[2], scratch[3]));
+}
+__device__ __forceinline__ float block_sum_256(float v, float* scratch) {
+    v = wave_sum(v);
+    __syncthreads();
+    if (threadIdx.x % WAVE == 0) scratch[threadIdx.x / WAVE] = v;
+    __syncthreads();
+    return (scratch[0] + scratch[1]) + (scratch[2] + scratch[3]);
+}
+
+__global__ __launch_bounds__(DEC_KEYS) void decode_scores_kernel(
+    const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_cache, float* __restrict__ S, float* __restrict__ ml,
+    const int* __restrict__ block_table, int max_blocks, const int* __restrict__ req_of_token, const int* __restrict__ positions,
+    int H, int Hkv, int hd, int page_size, int window, float scale, const float* __restrict__ slopes,
+    const float* __restrict__ log_r1, const float* __restrict__ log_r2, int n_parts) {
+    __shared__ float qs[DEC_HEADS * 256];
+    __shared__ float scratch[4];
+    const int t = blockIdx.x, kvh = blockIdx.y, part = blockIdx.z, tid = threadIdx.x;
+    const int G = H / Hkv;
+    const int pos = positions[t];
+    const int lo = (window > 0) ? max(0, pos - window + 1) : 0;
+    const int key = part * DEC_KEYS + tid;
+    const bool part_live = part * DEC_KEYS <= pos && part * DEC_KEYS + DEC_KEYS - 1 >= lo;
+    const bool valid = key >= lo && key <= pos;
+    const bf16_t* krow = k_cache;
+    if (valid) {
+        const long long page = block_table[(long long)req_of_token[t] * max_blocks + key / page_size];
+        krow = k_cache + ((page * Hkv + kvh) * page_size + key % page_size) * hd;
+    }
+    const float dist = (float)(pos - key);
+    for (int g0 = 0; g0 < G; g0 += DEC_HEADS) {
+        const int Gc = min(DEC_HEADS, G - g0);
+        const int head0 = kvh * G + g0;
+        if (!part_live) {                                       // uniform: no key of the part is visible
+            if (tid < Gc) {
+                float* dst = ml + (((long long)t * H + head0 + tid) * n_parts + part) * 2;
+                dst[0] = -INFINITY;
+                dst[1] = 0.f;
+            }
+            continue;
+        }
+        __syncthreads();
+        for (int i = tid; i < Gc * hd; i += DEC_KEYS) qs[i] = to_f32(q[((long long)t * H + head0) * hd + i]);
+        __syncthreads();
+        float acc[DEC_HEADS];
+#pragma unroll
+        for (int g = 0; g < DEC_HEADS; ++g) acc[g] = 0.f;
+        if (valid) {
+            for (int c = 0; c < hd; c += 8) {
+                const bf16x8 kv = *(const bf16x8*)(krow + c);
+                float kf[8];
+#pragma unroll
+                for (int e = 0; e < 8; ++e) kf[e] = (float)kv[e];
+#pragma unroll
+                for (int g = 0; g < DEC_HEADS; ++g) {
+                    if (g < Gc) {
+                        const float* qg = qs + g * hd + c;
+#pragma unroll
+                        for (int e = 0; e < 8; ++e) acc[g] = fmaf(qg[e], kf[e], acc[g]);
+                    }
+                }
+            }
+        }
+#pragma unroll
+        for (int g = 0; g < DEC_HEADS; ++g) {
+            if (g >= Gc) break;                                 // uniform
+            const int head = head0 + g;
+            float s = -INFINITY;
+            if (valid) {
+                s = acc[g] * scale;
+                if (slopes) s -= slopes[head] * dist;
+                if (log_r1) s -= log_r1[head] * log1pf(log_r2[head] * dist);
+                S[((long long)t * H + head) * n_parts * DEC_KEYS + key] = s;
+            }
+            const float m = block_max_256(s, scratch);
+            const float l = block_sum_256(valid ? expf(s - m) : 0.f, scratch);
+            if (tid == 0) {
+                float* dst = ml + (((long long)t * H + head) * n_parts + part) * 2;
+                dst[0] = m;
+                dst[1] = l;
+            }
+        }
+    }
+}
+
+__global__ __launch_bounds__(DEC_KEYS) void decode_values_kernel(
+    const float* __restrict__ S, const float* __restrict__ ml, const bf16_t* __restrict__ v_cache, float* __restrict__ po,
+    const int* __restrict__ block_table, int max_blocks, const int* __restrict__ req_of_token, const int* __restrict__ positions,
+    int H, int Hkv, int vd, int page_size, int window, const float* __restrict__ sinks, const float* __restrict__ talk, int n_parts) {
+    __shared__ float m_all[DEC_MAX_H], inv_all[DEC_MAX_H];
+    __shared__ float w[DEC_HEADS * DEC_KEYS];                 // weights [head of the group][key]; then the slices' sums
+    const int t = blockIdx.x, kvh = blockIdx.y, part = blockIdx.z, tid = threadIdx.x;
+    const int G = H / Hkv;
+    const int pos = positions[t];
+    const int lo = (window > 0) ? max(0, pos - window + 1) : 0;
+    if (part * DEC_KEYS > pos || part * DEC_KEYS + DEC_KEYS - 1 < lo) return;        // the merge skips such parts
+    const int key = part * DEC_KEYS + tid;
+    const bool valid = key >= lo && key <= pos;
+    const int* table = block_table + (long long)req_of_token[t] * max_blocks;
+    // every head's maximum and sum over the parts (all heads with a mixing matrix, else the group's)
+    const int h_first = talk ? 0 : kvh * G, h_count = talk ? H : G;
+    for (int i = tid; i < h_count; i += DEC_KEYS) {
+        const int head = h_first + i;
+        const float* src = ml + ((long long)t * H + head) * n_parts * 2;
+        float M = -INFINITY;
+        for (int p = 0; p < n_parts; ++p) M = fmaxf(M, src[2 * p]);
+        float L = 0.f;
+        for (int p = 0; p < n_parts; ++p) L += src[2 * p + 1] * expf(src[2 * p] - M);      // (a part without keys: 0 * exp(-inf) = 0)
+        if (sinks) {
+            const float sk = sinks[head], M2 = fmaxf(M, sk);
+            L = L * expf(M - M2) + expf(sk - M2);
+            M = M2;
+        }
+        m_all[i] = M;
+        inv_all[i] = 1.0f / L;
+    }
+    const int slices = max(1, DEC_KEYS / vd);                   // threads (channel, slice of the part's pages)
+    const int d = tid % vd, sl = tid / vd;
+    const bool works = tid < vd * slices;
+    const int first_page = part * DEC_KEYS / page_size;         // (DEC_KEYS is a multiple of the page size)
+    const int pages = DEC_KEYS / page_size;
+    for (int g0 = 0; g0 < G; g0 += DEC_HEADS) {
+        const int Gc = min(DEC_HEADS, G - g0);
+        const int head0 = kvh * G + g0;
+        __syncthreads();
+        // ---- the key's weights
+        float wk[DEC_HEADS];
+#pragma unroll
+        for (int g = 0; g < DEC_HEADS; ++g) wk[g] = 0.f;
+        if (valid) {
+            if (talk) {
+                for (int h2 = 0; h2 < H; ++h2) {
+                    const float e = expf(S[((long long)t * H + h2) * n_parts * DEC_KEYS + key] - m_all[h2]) * inv_all[h2];
+#pragma unroll
+                    for (int g = 0; g < DEC_HEADS; ++g)
+                        if (g < Gc) wk[g] = fmaf(talk[(head0 + g) * H + h2], e, wk[g]);
+                }
+            } else {
+#pragma unroll
+                for (int g = 0; g < DEC_HEADS; ++g)
+                    if (g < Gc) wk[g] = expf(S[((long long)t * H + head0 + g) * n_parts * DEC_KEYS + key] - m_all[g0 + g]) * inv_all[g0 + g];
+            }
+        }
+#pragma unroll
+        for (int g = 0; g < DEC_HEADS; ++g)
+            if (g < Gc) w[g * DEC_KEYS + tid] = wk[g];
+        __syncthreads();
+        // ---- weight * value
+        float acc[DEC_HEADS];
+#pragma unroll
+        for (int g = 0; g < DEC_HEADS; ++g) acc[g] = 0.f;
+        if (works) {
+            for (int pg = sl; pg < pages; pg += slices) {
+                const int key0 = (first_page + pg) * page_size;
+                if (key0 > pos || key0 + page_size - 1 < lo) continue;
+                const long long page = table[first_page + pg];
+                const bf16_t* vrow = v_cache + ((page * Hkv + kvh) * vd + d) * page_size;
+                for (int e0 = 0; e0 < page_size; e0 += 8) {
+                    const bf16x8 vv = *(const bf16x8*)(vrow + e0);
+                    const float* wrow = w + (pg * page_size + e0);
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) {
+                        // (positions after the last were never written: their weight is 0, but 0 * NaN is not)
+                        const float vf = key0 + e0 + e <= pos ? (float)vv[e] : 0.f;
+#pragma unroll
+                        for (int g = 0; g < DEC_HEADS; ++g)
+                            if (g < Gc) acc[g] = fmaf(wrow[g * DEC_KEYS + e], vf, acc[g]);
+                    }
+                }
+            }
+        }
+        __syncthreads();
+        if (works && sl > 0) {
+#pragma unroll
+            for (int g = 0; g < DEC_HEADS; ++g)
+                if (g < Gc) w[(g * slices + sl) * vd + d] = acc[g];
+        }
+        __syncthreads();
+        if (works && sl == 0) {
+#pragma unroll
+            for (int g = 0; g < DEC_HEADS; ++g) {
+                if (g < Gc) {
+                    float sum = acc[g];
+                    for (int s2 = 1; s2 < slices; ++s2) sum += w[(g * slices + s2) * vd + d];
+                    po[(((long long)t * H + head0 + g) * n_parts + part) * vd + d] = sum;
+                }
+            }
+        }
+    }
+}
+
+template <typename T>
+__global__ __launch_bounds__(WAVE) void decode_merge_kernel(const float* __restrict__ po, const int* __restrict__ positions,
+                                                            const float* __restrict__ gates, int gate_stride, T* __restrict__ out,
+                                                            int H, int vd, int window, int n_parts) {
+    const long long t = blockIdx.x;
+    const int head = blockIdx.y;
+    const int pos = positions[t];
+    const int lo = (window > 0) ? max(0, pos - window + 1) : 0;
+    const float g = gates ? 1.0f / (1.0f + expf(-gates[t * gate_stride + head])) : 1.f;
+    for (int d = threadIdx.x; d < vd; d += WAVE) {
+        float sum = 0.f;
+        for (int p = 0; p < n_parts; ++p) {
+            if (p * DEC_KEYS > pos || p * DEC_KEYS + DEC_KEYS - 1 < lo) continue;
+            sum += po[((t * H + head) * n_parts + p) * vd + d];
+        }
+        out[(t * H + head) * vd + d] = from_f32<T>(sum * g);
+    }
+}
+}  // namespace
+
+// Single tokens, bfloat16 q and caches, float32 weights.  S float32 [tokens * H * n_parts * 256], ml float32
+// [tokens * H * n_parts * 2] and po float32 [tokens * H * n_parts * vd] are work space; n_parts * 256 covers every position + 1.
+// talk float32 [H][H] or null; gates float32 (row stride gate_stride) or null; out_dt: type of out [tokens][H][vd].
+TUFF_EXPORT int tuff_attention_decode_exact(const void* q, const void* k_cache, const void* v_cache, void* out, int out_dt,
+                                            float* S, float* ml, float* po, const int* block_table, int max_blocks,
+                                            const int* req_of_token, const int* positions, int n_tokens, int H, int Hkv, int hd,
+                                            int vd, int page_size, int window, float scale, const float* sinks, const float* slopes,
+                                            const float* log_r1, const float* log_r2, const float* talk, const float* gates,
+                                            int gate_stride, int n_parts, hipStream_t stream) {
+    if (n_tokens <= 0) return 0;
+    if (Hkv <= 0 || H % Hkv != 0 || H > DEC_MAX_H || hd % 8 != 0 || hd > 256 || vd <= 0 || vd > DEC_KEYS) return -2;
+    if (page_size % 8 != 0 || DEC_KEYS % page_size != 0 || n_parts <= 0 || n_parts > 65535 || Hkv > 65535) return -2;
+    if ((log_r1 == nullptr) != (log_r2 == nullptr) || !S || !ml || !po) return -2;
+    dim3 grid(n_tokens, Hkv, n_parts), block(DEC_KEYS);
+    hipLaunchKernelGGL(decode_scores_kernel, grid, block, 0, stream, (const bf16_t*)q, (const bf16_t*)k_cache, S, ml, block_table,
+                       max_blocks, req_of_token, positions, H, Hkv, hd, page_size, window, scale, slopes, log_r1, log_r2, n_parts);
+    hipLaunchKernelGGL(decode_values_kernel, grid, block, 0, stream, (const float*)S, (const float*)ml, (const bf16_t*)v_cache, po,
+                       block_table, max_blocks, req_of_token, positions, H, Hkv, vd, page_size, window, sinks, talk, n_parts);
+    dim3 mgrid(n_tokens, H), mblock(WAVE);
+    if (out_dt == DT_F32)
+        hipLaunchKernelGGL(decode_merge_kernel<float>, mgrid, mblock, 0, stream, (const float*)po, positions, gates, gate_stride,
+                           (float*)out, H, vd, window, n_parts);
+    else
+        hipLaunchKernelGGL(decode_merge_kernel<bf16_t>, mgrid, mblock, 0, stream, (const float*)po, positions, gates, gate_stride,
+                           (bf16_t*)out, H, vd, window, n_parts);
+    return launch_status();
+}

@@ -100,6 +100,10 @@ _SIGNATURES = {
         "tuff_attention_general": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_void_p, _c_int,
                                    _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
                                    _c_float, _c_void_p, _c_void_p, _c_int, _c_void_p, _c_void_p, _c_int, _c_void_p],
+        "tuff_attention_decode_exact": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_void_p, _c_void_p, _c_void_p,
+                                        _c_void_p, _c_int, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
+                                        _c_int, _c_float, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p,
+                                        _c_int, _c_int, _c_void_p],
         "tuff_head_mix_gate": [_c_void_p, _c_int, _c_void_p, _c_void_p, _c_int, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int,
                                _c_void_p],
     },
@@ -1250,6 +1254,67 @@ def attention_prefill(q, k_cache, v_cache, out, *, block_table, blocks, req_info
         _check(load("attention_prefill").tuff_attention_prefill_sinks(*args, sinks.data_ptr(), _stream()), "attention_prefill")
         if merge is not None:
             _check(load("attention_mfma").tuff_attention_merge_sinks(*merge, sinks.data_ptr(), _stream()), "attention_merge")
+
+
+DECODE_EXACT_KEYS = 256          # keys a part of attention_decode_exact
+
+
+def attention_decode_exact_supported(dtype, H: int, hd: int, vd: int, page_size: int) -> bool:
+    return (dtype == torch.bfloat16 and H <= 256 and hd % 8 == 0 and hd <= 256 and 1 <= vd <= DECODE_EXACT_KEYS
+            and page_size % 8 == 0 and DECODE_EXACT_KEYS % page_size == 0)
+
+
+def attention_decode_exact(q, k_cache, v_cache, out, *, block_table, req_of_token, positions, H, Hkv, hd, vd, page_size,
+                           max_ctx_len, window=0, scale=None, sinks=None, slopes=None, log_distance=None, talk=None,
+                           gates=None) -> None:
+    """Single tokens over the bfloat16 cache with float32 softmax weights: the scores of parts of 256 keys (a key's row
+    read once for all heads of its kv group), then the normalised weights on the values (read once too), then the sum over
+    the parts.  log_distance = (r1, r2): r1[h] * ln(1 + r2[h] * (position - key)) is taken off the scaled scores.
+    talk float32 [H, H]: head h's weights are sum_g talk[h, g] weights_g, on the values of h's own kv head.
+    gates float32 [T, >= H] (a row may be wider): out[t, h] is multiplied by sigmoid(gates[t, h]).
+    out [T, H * vd], bfloat16 or float32."""
+    T = q.shape[0]
+    if not attention_decode_exact_supported(q.dtype, H, hd, vd, page_size):
+        raise KernelError(f"attention_decode_exact: bfloat16, heads {H} <= 256, key size {hd} a multiple of 8, "
+                          f"value size {vd} <= 256, page size {page_size} a divisor of 256")
+    _gpu("q", q, torch.bfloat16, (T, H * hd))
+    _gpu("out", out, shape=(T, H * vd))
+    P = k_cache.shape[0]
+    _gpu("k_cache", k_cache, torch.bfloat16, (P, Hkv, page_size, hd))
+    _gpu("v_cache", v_cache, torch.bfloat16, (P, Hkv, vd, page_size))
+    _opt("sinks", sinks, torch.float32, (H,))
+    _opt("slopes", slopes, torch.float32, (H,))
+    _opt("talk", talk, torch.float32, (H, H))
+    r1 = r2 = None
+    if log_distance is not None:
+        r1, r2 = log_distance
+        _gpu("log_distance r1", r1, torch.float32, (H,))
+        _gpu("log_distance r2", r2, torch.float32, (H,))
+    gate_stride = 0
+    if gates is not None:
+        _gpu("gates", gates, torch.float32)
+        if gates.dim() != 2 or gates.shape[0] != T or gates.shape[1] < H or gates.stride(1) != 1:
+            raise KernelError("attention_decode_exact: gates must be float32 [tokens, >= heads]")
+        gate_stride = gates.stride(0)
+    _gpu("block_table", block_table, torch.int32)
+    if block_table.dim() != 2 or block_table.shape[1] * page_size < int(max_ctx_len):
+        raise KernelError("attention_decode_exact: block_table must be [requests, blocks] and cover the longest context")
+    _gpu("req_of_token", req_of_token, torch.int32, (T,))
+    _gpu("positions", positions, torch.int32, (T,))
+    if H % Hkv:
+        raise KernelError("attention_decode_exact: the query heads must be a multiple of the kv heads")
+    if scale is None:
+        scale = 1.0 / math.sqrt(hd)
+    n_parts = max(1, -(-int(max_ctx_len) // DECODE_EXACT_KEYS))
+    S = torch.empty(T * H * n_parts * DECODE_EXACT_KEYS, dtype=torch.float32, device=q.device)
+    ml = torch.empty(T * H * n_parts * 2, dtype=torch.float32, device=q.device)
+    po = torch.empty(T * H * n_parts * vd, dtype=torch.float32, device=q.device)
+    ptr = lambda x: None if x is None else x.data_ptr()
+    _check(load("attention").tuff_attention_decode_exact(
+        q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), out.data_ptr(), _dt(out), S.data_ptr(), ml.data_ptr(), po.data_ptr(),
+        block_table.data_ptr(), block_table.shape[1], req_of_token.data_ptr(), positions.data_ptr(), T, H, Hkv, hd, vd, page_size,
+        int(window or 0), float(scale), ptr(sinks), ptr(slopes), ptr(r1), ptr(r2), ptr(talk), ptr(gates), gate_stride, n_parts,
+        _stream()), "attention_decode_exact")
 
 
 def attention_prefill_wide_supported(dtype, hd: int, vd: int, page_size: int) -> bool:

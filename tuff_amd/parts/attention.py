@@ -74,10 +74,25 @@ class PagedAttention:
             ctx.host[key] = runs
         return runs
 
-    def attend(self, q, o, ctx, cache, g) -> None:
+    def _single_tokens_exact(self, dtype, ctx, page_size) -> bool:
+        """A step of single tokens whose weights stay float32: the kernels that read a request's keys and values once
+        for all heads, and mix and gate the heads themselves."""
+        special = (getattr(self, "log_distance", None) is not None or getattr(self, "talk", None) is not None
+                   or getattr(self, "exact_weights", False))
+        return (special and ctx.max_q_len == 1
+                and ops.attention_decode_exact_supported(dtype, self.H, self.hd, self.vd, page_size))
+
+    def attend(self, q, o, ctx, cache, g, gates=None) -> None:
         G = self.H // self.Hkv
         log_distance, talk = getattr(self, "log_distance", None), getattr(self, "talk", None)
         exact = getattr(self, "exact_weights", False)
+        if self._single_tokens_exact(q.dtype, ctx, cache.page_size):
+            ops.attention_decode_exact(q, cache.k, cache.v, o, block_table=g.block_table, req_of_token=ctx.req_of_token,
+                                       positions=ctx.positions, H=self.H, Hkv=self.Hkv, hd=self.hd, vd=self.vd,
+                                       page_size=cache.page_size, max_ctx_len=ctx.max_ctx_len, window=self.window or 0,
+                                       scale=self.scale, sinks=self.sinks, slopes=self.slopes, log_distance=log_distance,
+                                       talk=talk, gates=gates)
+            return
         if ((log_distance is not None or talk is not None or exact) and ctx.max_q_len > 1
                 and ops.attention_prefill_wide_supported(q.dtype, self.hd, self.vd, cache.page_size)):
             # prompt portions in the step: the matrix-core kernel in its wide form (single tokens beside them are blocks
@@ -275,7 +290,10 @@ class AttentionMixer(Mixer, PagedAttention):
                          state_slot=ctx.state_slot, q_len=ctx.q_len, activation=None)
         q = self.rt.empty(T, H * hd) if vd == hd else None
         # (with mixed heads: every head's weights on every kv head's values, float32, for the kernel that mixes them)
-        o = self.rt.empty(T, H * vd) if self.talk is None else torch.empty(T, H * Hkv * vd, dtype=torch.float32, device=qkv.device)
+        # (single tokens with float32 weights: the attention kernels mix and gate the heads themselves)
+        finished = self._single_tokens_exact(qkv.dtype, ctx, cache.page_size)
+        o = (self.rt.empty(T, H * vd) if self.talk is None or finished
+             else torch.empty(T, H * Hkv * vd, dtype=torch.float32, device=qkv.device))
         norm = dict(eps=self.eps or 0.0, q_norm_w=self.q_norm_w, k_norm_w=self.k_norm_w)
         tables = self.position.rotary_tables() if self.position is not None else None
         fused = self.position is None or tables is not None
@@ -301,7 +319,7 @@ class AttentionMixer(Mixer, PagedAttention):
                 if write_cache:
                     ops.kv_write(kk, qkv[:, (H + Hkv) * hd:].contiguous(),
                                  cache.k, cache.v, g.slot_mapping, Hkv=Hkv, hd=hd, vd=vd, page_size=cache.page_size)
-                self.attend(qq, o, ctx, cache, g)
+                self.attend(qq, o, ctx, cache, g, gates)
                 return
             if one_kernel:
                 # single tokens, heads of 64: norm, rotation, cache write and attention in one kernel
@@ -327,11 +345,11 @@ class AttentionMixer(Mixer, PagedAttention):
                 if write_cache:
                     v = qkv[:, (H + Hkv) * hd:].contiguous()
                     ops.kv_write(k, v, cache.k, cache.v, g.slot_mapping, Hkv=Hkv, hd=hd, page_size=cache.page_size)
-            self.attend(q, o, ctx, cache, g)
+            self.attend(q, o, ctx, cache, g, gates)
 
         ctx.run_eagerly(over_the_cache)
         heads = o             # (over_the_cache keeps `o` for its replays: the name is not bound anew)
-        if self.talk is not None or gates is not None:
+        if not finished and (self.talk is not None or gates is not None):
             heads = self.rt.empty(T, H * vd)
             ops.head_mix_gate(o, heads, H=H, Hkv=Hkv, vd=vd, talk=self.talk, gates=gates)
         self.out.forward(heads, accumulate_into=residual, next_norm=next_norm)
