@@ -374,13 +374,34 @@ def kugalorn_config(size: str):
                              "layers": [kinds[i % 2] for i in range(L)]})
 
 
-def lfm2_config_like(size: str):
+def loluzen_config(size: str):
+    """`--design loluzen`: layers take turns between a pair (attention with biases, a logarithmic distance penalty and
+    mixed heads, heads of 64, beside a forget-gate recurrence with keys of 64 and values of 128 a head) and attention
+    behind convolutions of 4 taps (heads of 64, half of a head's channels rotated), every layer with a dense
+    squared-relu feed-forward."""
+    from tuff_amd.models.registry import config_from_dict
+    d, L, H, G, ff, _, _, _ = DESIGN_SIZES[size]
+    dense = {"kind": "dense", "ff": ff}
+    kinds = [
+        {"type": "parallel", "mixer": {"left": {"heads": H, "kv_heads": G, "dim": 64, "vdim": 64, "scale": 0.125},
+                                       "right": {"heads": d // 128, "dim": 64, "vdim": 128}}, "mlp": dense},
+        {"type": "attention", "mixer": {"heads": H, "kv_heads": G, "dim": 64, "vdim": 64, "scale": 0.125, "conv": 4,
+                                        "rot": {"base": 10000.0, "dims": 32,
+                                                "scaling": {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 8192}}}, "mlp": dense},
+    ]
+    return config_from_dict({"architecture": "Loluzen", "vocab": DESIGN_VOCAB, "width": d, "embedding": {"scale": 1.0},
+                             "norm": {"eps": 1e-5}, "residual_mult": 0.5, "layers": [kinds[i % 2] for i in range(L)]})
+
+
+def lfm2_config_like(size: str, attention_every: int = 4):
     """The LFM2 model of the same width, depth, heads, vocabulary and dense feed-forward: its short-conv
-    layers stand where the other design has its recurrences."""
+    layers stand where the other design has its recurrences (attention_every 1: attention in every layer, beside a
+    design that has it in every layer)."""
     from tuff_amd.models.registry import config_from_dict
     d, L, H, G, ff, _, _, _ = DESIGN_SIZES[size]
     return config_from_dict(dict(
-        architectures=["Lfm2ForCausalLM"], num_hidden_layers=L, full_attn_idxs=[i for i in range(L) if i % 4 == 1],
+        architectures=["Lfm2ForCausalLM"], num_hidden_layers=L,
+        full_attn_idxs=[i for i in range(L) if attention_every == 1 or i % attention_every == 1],
         hidden_size=d, num_attention_heads=H, num_key_value_heads=G, block_ff_dim=ff, block_auto_adjust_ff_dim=False,
         vocab_size=DESIGN_VOCAB, rope_theta=1000000.0, conv_L_cache=3, norm_eps=1e-5, tie_word_embeddings=False,
         max_position_embeddings=32768))
@@ -452,17 +473,18 @@ def time_design(cfg, dtype: str, prefill_tokens: int, batch: int, context: int, 
 
 
 def run_design(args) -> dict:
-    """`--design pafodra|kugalorn`: that decoder at sizes that resemble a real model's layers (random weights)
+    """`--design pafodra|kugalorn|loluzen`: that decoder at sizes that resemble a real model's layers (random weights)
     beside the LFM2 decoder of equal width, depth and feed-forward."""
     dtype = "bfloat16" if args.dtype == "bf16" else "float32"
     classes = os.environ.get("TUFF_TRACE", "")[:1] == "1"
-    design, make = args.design, {"pafodra": pafodra_config, "kugalorn": kugalorn_config}[args.design]
+    design, make = args.design, {"pafodra": pafodra_config, "kugalorn": kugalorn_config, "loluzen": loluzen_config}[args.design]
+    every = 1 if design == "loluzen" else 4
     out = {"design": design, "dtype": args.dtype, "prefill_tokens": PREFILL_TOKENS, "decode_batch": args.batch,
            "decode_context": args.design_context, "data": f"synthetic: seeded random weights (seed {SEED}), uniform random token ids",
            "sizes": {}}
     for size in args.design_sizes.split(","):
         rec = {}
-        for name, cfg in ((design, make(size)), ("lfm2", lfm2_config_like(size))):
+        for name, cfg in ((design, make(size)), ("lfm2", lfm2_config_like(size, every))):
             rec[name] = time_design(cfg, dtype, PREFILL_TOKENS, args.batch, args.design_context, args.point_steps, classes)
         rec["prefill_ratio"] = round(rec[design]["prefill_tok_s"] / rec["lfm2"]["prefill_tok_s"], 3)
         rec["decode_ratio"] = round(rec[design]["decode_tok_s"] / rec["lfm2"]["decode_tok_s"], 3)
@@ -548,7 +570,7 @@ def main() -> int:
     ap.add_argument("--shape", default="1.2b", choices=["1.2b"] + sorted(OTHER_SHAPES),
                     help="measure another shape of the architecture in the benchmark's place (for profiling; "
                          "its points only, no other shapes after it)")
-    ap.add_argument("--design", choices=["pafodra", "kugalorn"],
+    ap.add_argument("--design", choices=["pafodra", "kugalorn", "loluzen"],
                     help="instead of the benchmark: prefill and decode of another design at sizes that resemble a real "
                          "model's layers, beside the LFM2 model of equal size (TUFF_TRACE=1 adds GPU time by kernel class)")
     ap.add_argument("--design-sizes", default="1k,2k", help="with --design: which of " + ",".join(sorted(DESIGN_SIZES)))
