@@ -230,7 +230,7 @@ __global__ __launch_bounds__(DEC_KEYS) void decode_scores_kernel(
     __shared__ float scratch[4];
     const int t = blockIdx.x, kvh = blockIdx.y, part = blockIdx.z, tid = threadIdx.x;
     const int G = H / Hkv;
-    const int pos = positions[t];
+    const int pos = positions[blockIdx.x];
     const int lo = (window > 0) ? max(0, pos - window + 1) : 0;
     const int key = part * DEC_KEYS + tid;
     const bool part_live = part * DEC_KEYS <= pos && part * DEC_KEYS + DEC_KEYS - 1 >= lo;
@@ -259,17 +259,27 @@ __global__ __launch_bounds__(DEC_KEYS) void decode_scores_kernel(
 #pragma unroll
         for (int g = 0; g < DEC_HEADS; ++g) acc[g] = 0.f;
         if (valid) {
-            for (int c = 0; c < hd; c += 8) {
-                const bf16x8 kv = *(const bf16x8*)(krow + c);
-                float kf[8];
+            for (int c0 = 0; c0 < hd; c0 += 32) {            // four pieces of the row are loaded before any is used
+                bf16x8 kv[4];
 #pragma unroll
-                for (int e = 0; e < 8; ++e) kf[e] = (float)kv[e];
+                for (int u = 0; u < 4; ++u) {
+                    const bf16x8 z = {0, 0, 0, 0, 0, 0, 0, 0};
+                    kv[u] = c0 + 8 * u < hd ? *(const bf16x8*)(krow + c0 + 8 * u) : z;
+                }
 #pragma unroll
-                for (int g = 0; g < DEC_HEADS; ++g) {
-                    if (g < Gc) {
-                        const float* qg = qs + g * hd + c;
+                for (int u = 0; u < 4; ++u) {
+                    const int c = c0 + 8 * u;
+                    if (c >= hd) break;
+                    float kf[8];
 #pragma unroll
-                        for (int e = 0; e < 8; ++e) acc[g] = fmaf(qg[e], kf[e], acc[g]);
+                    for (int e = 0; e < 8; ++e) kf[e] = (float)kv[u][e];
+#pragma unroll
+                    for (int g = 0; g < DEC_HEADS; ++g) {
+                        if (g < Gc) {
+                            const float* qg = qs + g * hd + c;
+#pragma unroll
+                            for (int e = 0; e < 8; ++e) acc[g] = fmaf(qg[e], kf[e], acc[g]);
+                        }
                     }
                 }
             }
@@ -304,7 +314,7 @@ __global__ __launch_bounds__(DEC_KEYS) void decode_values_kernel(
     __shared__ float w[DEC_HEADS * DEC_KEYS];                 // weights [head of the group][key]; then the slices' sums
     const int t = blockIdx.x, kvh = blockIdx.y, part = blockIdx.z, tid = threadIdx.x;
     const int G = H / Hkv;
-    const int pos = positions[t];
+    const int pos = positions[blockIdx.x];
     const int lo = (window > 0) ? max(0, pos - window + 1) : 0;
     if (part * DEC_KEYS > pos || part * DEC_KEYS + DEC_KEYS - 1 < lo) return;        // the merge skips such parts
     const int key = part * DEC_KEYS + tid;
@@ -312,26 +322,39 @@ __global__ __launch_bounds__(DEC_KEYS) void decode_values_kernel(
     const int* table = block_table + (long long)req_of_token[t] * max_blocks;
     // every head's maximum and sum over the parts (all heads with a mixing matrix, else the group's)
     const int h_first = talk ? 0 : kvh * G, h_count = talk ? H : G;
-    for (int i = tid; i < h_count; i += DEC_KEYS) {
-        const int head = h_first + i;
-        const float* src = ml + ((long long)t * H + head) * n_parts * 2;
-        float M = -INFINITY;
-        for (int p = 0; p < n_parts; ++p) M = fmaxf(M, src[2 * p]);
-        float L = 0.f;
-        for (int p = 0; p < n_parts; ++p) L += src[2 * p + 1] * expf(src[2 * p] - M);      // (a part without keys: 0 * exp(-inf) = 0)
+    // (eight lanes a head, each a share of the parts, so that the loads are in flight together)
+    for (int i0 = 0; i0 < h_count; i0 += DEC_KEYS / 8) {
+        const int i = i0 + tid / 8, sub = tid % 8;
+        const bool live = i < h_count;
+        const int head = h_first + (live ? i : 0);
+        const float2* src = (const float2*)(ml + ((long long)t * H + head) * n_parts * 2);
+        float M = -INFINITY, L = 0.f;
+        for (int p = sub; p < n_parts; p += 8) {
+            const float2 v = src[p];
+            const float M2 = fmaxf(M, v.x);
+            if (M2 > -INFINITY) L = L * expf(M - M2) + v.y * expf(v.x - M2);             // (a part without keys: -inf, 0)
+            M = M2;
+        }
+#pragma unroll
+        for (int off = 1; off < 8; off *= 2) {
+            const float Mo = __shfl_xor(M, off, WAVE), Lo = __shfl_xor(L, off, WAVE);
+            const float M2 = fmaxf(M, Mo);
+            if (M2 > -INFINITY) L = L * expf(M - M2) + Lo * expf(Mo - M2);
+            M = M2;
+        }
         if (sinks) {
             const float sk = sinks[head], M2 = fmaxf(M, sk);
             L = L * expf(M - M2) + expf(sk - M2);
             M = M2;
         }
-        m_all[i] = M;
-        inv_all[i] = 1.0f / L;
+        if (live && sub == 0) {
+            m_all[i] = M;
+            inv_all[i] = 1.0f / L;
+        }
     }
     const int slices = max(1, DEC_KEYS / vd);                   // threads (channel, slice of the part's pages)
     const int d = tid % vd, sl = tid / vd;
     const bool works = tid < vd * slices;
-    const int first_page = part * DEC_KEYS / page_size;         // (DEC_KEYS is a multiple of the page size)
-    const int pages = DEC_KEYS / page_size;
     for (int g0 = 0; g0 < G; g0 += DEC_HEADS) {
         const int Gc = min(DEC_HEADS, G - g0);
         const int head0 = kvh * G + g0;
@@ -342,11 +365,20 @@ __global__ __launch_bounds__(DEC_KEYS) void decode_values_kernel(
         for (int g = 0; g < DEC_HEADS; ++g) wk[g] = 0.f;
         if (valid) {
             if (talk) {
-                for (int h2 = 0; h2 < H; ++h2) {
-                    const float e = expf(S[((long long)t * H + h2) * n_parts * DEC_KEYS + key] - m_all[h2]) * inv_all[h2];
+                for (int h0 = 0; h0 < H; h0 += 8) {          // eight heads' scores are loaded before any is used
+                    float sv[8];
 #pragma unroll
-                    for (int g = 0; g < DEC_HEADS; ++g)
-                        if (g < Gc) wk[g] = fmaf(talk[(head0 + g) * H + h2], e, wk[g]);
+                    for (int u = 0; u < 8; ++u)
+                        sv[u] = h0 + u < H ? S[((long long)t * H + h0 + u) * n_parts * DEC_KEYS + key] : -INFINITY;
+#pragma unroll
+                    for (int u = 0; u < 8; ++u) {
+                        const int h2 = h0 + u;
+                        if (h2 >= H) break;
+                        const float e = expf(sv[u] - m_all[h2]) * inv_all[h2];
+#pragma unroll
+                        for (int g = 0; g < DEC_HEADS; ++g)
+                            if (g < Gc) wk[g] = fmaf(talk[(head0 + g) * H + h2], e, wk[g]);
+                    }
                 }
             } else {
 #pragma unroll
@@ -363,18 +395,35 @@ __global__ __launch_bounds__(DEC_KEYS) void decode_values_kernel(
 #pragma unroll
         for (int g = 0; g < DEC_HEADS; ++g) acc[g] = 0.f;
         if (works) {
-            for (int pg = sl; pg < pages; pg += slices) {
-                const int key0 = (first_page + pg) * page_size;
-                if (key0 > pos || key0 + page_size - 1 < lo) continue;
-                const long long page = table[first_page + pg];
-                const bf16_t* vrow = v_cache + ((page * Hkv + kvh) * vd + d) * page_size;
-                for (int e0 = 0; e0 < page_size; e0 += 8) {
-                    const bf16x8 vv = *(const bf16x8*)(vrow + e0);
-                    const float* wrow = w + (pg * page_size + e0);
+            // pieces of 8 keys; the page numbers and then the values of four pieces are loaded before any is used
+            constexpr int PIECES = DEC_KEYS / 8;
+            for (int c0 = sl; c0 < PIECES; c0 += 4 * slices) {
+                const bf16_t* src[4];
+                bool live[4];
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    const int piece = c0 + u * slices;
+                    const int key0 = part * DEC_KEYS + piece * 8;
+                    live[u] = piece < PIECES && key0 <= pos && key0 + 7 >= lo;
+                    const long long page = live[u] ? table[key0 / page_size] : 0;
+                    src[u] = v_cache + ((page * Hkv + kvh) * vd + d) * page_size + key0 % page_size;
+                }
+                bf16x8 vv[4];
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    const bf16x8 z = {0, 0, 0, 0, 0, 0, 0, 0};
+                    vv[u] = live[u] ? *(const bf16x8*)src[u] : z;
+                }
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    if (!live[u]) continue;
+                    const int piece = c0 + u * slices;
+                    const int key0 = part * DEC_KEYS + piece * 8;
+                    const float* wrow = w + piece * 8;
 #pragma unroll
                     for (int e = 0; e < 8; ++e) {
                         // (positions after the last were never written: their weight is 0, but 0 * NaN is not)
-                        const float vf = key0 + e0 + e <= pos ? (float)vv[e] : 0.f;
+                        const float vf = key0 + e <= pos ? (float)vv[u][e] : 0.f;
 #pragma unroll
                         for (int g = 0; g < DEC_HEADS; ++g)
                             if (g < Gc) acc[g] = fmaf(wrow[g * DEC_KEYS + e], vf, acc[g]);
@@ -408,7 +457,7 @@ __global__ __launch_bounds__(WAVE) void decode_merge_kernel(const float* __restr
                                                             int H, int vd, int window, int n_parts) {
     const long long t = blockIdx.x;
     const int head = blockIdx.y;
-    const int pos = positions[t];
+    const int pos = positions[blockIdx.x];
     const int lo = (window > 0) ? max(0, pos - window + 1) : 0;
     const float g = gates ? 1.0f / (1.0f + expf(-gates[t * gate_stride + head])) : 1.f;
     for (int d = threadIdx.x; d < vd; d += WAVE) {
