@@ -200,7 +200,7 @@ TUFF_EXPORT int tuff_head_mix_gate(const void* o, int in_dt, const float* talk, 
 //            matrix, sum_g talk[h][g] w_g from the weights of all heads; then the threads, each a value channel and
 //            a share of the part's pages, sum weight * value for the group's heads; partial sums per part go to po.
 //   merge    out[token][head] = gate * sum over the parts that hold a visible key.
-// Heads are taken sixteen at a time.  Layouts as above: K [page][kv head][offset][hd], V [page][kv head][vd][offset].
+// Heads are taken sixteen at a time (or as many as the group has, rounded up to a power of two).  Layouts as above: K [page][kv head][offset][hd], V [page][kv head][vd][offset].
 namespace {
 constexpr int DEC_KEYS = 256;         // keys a part, threads a workgroup
 constexpr int DEC_HEADS = 16;         // heads of a group taken together
@@ -221,6 +221,7 @@ __device__ __forceinline__ float block_sum_256(float v, float* scratch) {
     return (scratch[0] + scratch[1]) + (scratch[2] + scratch[3]);
 }
 
+template <int GC>
 __global__ __launch_bounds__(DEC_KEYS) void decode_scores_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_cache, float* __restrict__ S, float* __restrict__ ml,
     const int* __restrict__ block_table, int max_blocks, const int* __restrict__ req_of_token, const int* __restrict__ positions,
@@ -241,8 +242,8 @@ __global__ __launch_bounds__(DEC_KEYS) void decode_scores_kernel(
         krow = k_cache + ((page * Hkv + kvh) * page_size + key % page_size) * hd;
     }
     const float dist = (float)(pos - key);
-    for (int g0 = 0; g0 < G; g0 += DEC_HEADS) {
-        const int Gc = min(DEC_HEADS, G - g0);
+    for (int g0 = 0; g0 < G; g0 += GC) {
+        const int Gc = min(GC, G - g0);
         const int head0 = kvh * G + g0;
         if (!part_live) {                                       // uniform: no key of the part is visible
             if (tid < Gc) {
@@ -255,9 +256,9 @@ __global__ __launch_bounds__(DEC_KEYS) void decode_scores_kernel(
         __syncthreads();
         for (int i = tid; i < Gc * hd; i += DEC_KEYS) qs[i] = to_f32(q[((long long)t * H + head0) * hd + i]);
         __syncthreads();
-        float acc[DEC_HEADS];
+        float acc[GC];
 #pragma unroll
-        for (int g = 0; g < DEC_HEADS; ++g) acc[g] = 0.f;
+        for (int g = 0; g < GC; ++g) acc[g] = 0.f;
         if (valid) {
             for (int c0 = 0; c0 < hd; c0 += 32) {            // four pieces of the row are loaded before any is used
                 bf16x8 kv[4];
@@ -274,18 +275,16 @@ __global__ __launch_bounds__(DEC_KEYS) void decode_scores_kernel(
 #pragma unroll
                     for (int e = 0; e < 8; ++e) kf[e] = (float)kv[u][e];
 #pragma unroll
-                    for (int g = 0; g < DEC_HEADS; ++g) {
-                        if (g < Gc) {
-                            const float* qg = qs + g * hd + c;
+                    for (int g = 0; g < GC; ++g) {                  // (g >= Gc: whatever LDS holds, never stored)
+                        const float* qg = qs + g * hd + c;
 #pragma unroll
-                            for (int e = 0; e < 8; ++e) acc[g] = fmaf(qg[e], kf[e], acc[g]);
-                        }
+                        for (int e = 0; e < 8; ++e) acc[g] = fmaf(qg[e], kf[e], acc[g]);
                     }
                 }
             }
         }
 #pragma unroll
-        for (int g = 0; g < DEC_HEADS; ++g) {
+        for (int g = 0; g < GC; ++g) {
             if (g >= Gc) break;                                 // uniform
             const int head = head0 + g;
             float s = -INFINITY;
@@ -306,6 +305,7 @@ __global__ __launch_bounds__(DEC_KEYS) void decode_scores_kernel(
     }
 }
 
+template <int GC>
 __global__ __launch_bounds__(DEC_KEYS) void decode_values_kernel(
     const float* __restrict__ S, const float* __restrict__ ml, const bf16_t* __restrict__ v_cache, float* __restrict__ po,
     const int* __restrict__ block_table, int max_blocks, const int* __restrict__ req_of_token, const int* __restrict__ positions,
@@ -320,6 +320,17 @@ __global__ __launch_bounds__(DEC_KEYS) void decode_values_kernel(
     const int key = part * DEC_KEYS + tid;
     const bool valid = key >= lo && key <= pos;
     const int* table = block_table + (long long)req_of_token[t] * max_blocks;
+    // What depends on nothing the kernel computes is asked for first, so that memory is waited for once: the part's page
+    // numbers (into LDS), and without a mixing matrix the key's scores for the first heads of the group.
+    __shared__ int page_of[DEC_KEYS / 8];
+    if (tid < DEC_KEYS / page_size) {
+        const int key0 = part * DEC_KEYS + tid * page_size;
+        page_of[tid] = (key0 <= pos && key0 + page_size - 1 >= lo) ? table[key0 / page_size] : 0;
+    }
+    float s_first[GC];
+#pragma unroll
+    for (int g = 0; g < GC; ++g)
+        s_first[g] = (!talk && valid && g < G) ? S[((long long)t * H + kvh * G + g) * n_parts * DEC_KEYS + key] : -INFINITY;
     // every head's maximum and sum over the parts (all heads with a mixing matrix, else the group's)
     const int h_first = talk ? 0 : kvh * G, h_count = talk ? H : G;
     // (eight lanes a head, each a share of the parts, so that the loads are in flight together)
@@ -355,14 +366,14 @@ __global__ __launch_bounds__(DEC_KEYS) void decode_values_kernel(
     const int slices = max(1, DEC_KEYS / vd);                   // threads (channel, slice of the part's pages)
     const int d = tid % vd, sl = tid / vd;
     const bool works = tid < vd * slices;
-    for (int g0 = 0; g0 < G; g0 += DEC_HEADS) {
-        const int Gc = min(DEC_HEADS, G - g0);
+    for (int g0 = 0; g0 < G; g0 += GC) {
+        const int Gc = min(GC, G - g0);
         const int head0 = kvh * G + g0;
         __syncthreads();
         // ---- the key's weights
-        float wk[DEC_HEADS];
+        float wk[GC];
 #pragma unroll
-        for (int g = 0; g < DEC_HEADS; ++g) wk[g] = 0.f;
+        for (int g = 0; g < GC; ++g) wk[g] = 0.f;
         if (valid) {
             if (talk) {
                 for (int h0 = 0; h0 < H; h0 += 8) {          // eight heads' scores are loaded before any is used
@@ -376,24 +387,26 @@ __global__ __launch_bounds__(DEC_KEYS) void decode_values_kernel(
                         if (h2 >= H) break;
                         const float e = expf(sv[u] - m_all[h2]) * inv_all[h2];
 #pragma unroll
-                        for (int g = 0; g < DEC_HEADS; ++g)
-                            if (g < Gc) wk[g] = fmaf(talk[(head0 + g) * H + h2], e, wk[g]);
+                        for (int g = 0; g < GC; ++g) wk[g] = fmaf(talk[min(head0 + g, H - 1) * H + h2], e, wk[g]);
                     }
                 }
             } else {
 #pragma unroll
-                for (int g = 0; g < DEC_HEADS; ++g)
-                    if (g < Gc) wk[g] = expf(S[((long long)t * H + head0 + g) * n_parts * DEC_KEYS + key] - m_all[g0 + g]) * inv_all[g0 + g];
+                for (int g = 0; g < GC; ++g)
+                    if (g < Gc) {
+                        const float sc = g0 == 0 ? s_first[g] : S[((long long)t * H + head0 + g) * n_parts * DEC_KEYS + key];
+                        wk[g] = expf(sc - m_all[g0 + g]) * inv_all[g0 + g];
+                    }
             }
         }
 #pragma unroll
-        for (int g = 0; g < DEC_HEADS; ++g)
+        for (int g = 0; g < GC; ++g)
             if (g < Gc) w[g * DEC_KEYS + tid] = wk[g];
         __syncthreads();
         // ---- weight * value
-        float acc[DEC_HEADS];
+        float acc[GC];
 #pragma unroll
-        for (int g = 0; g < DEC_HEADS; ++g) acc[g] = 0.f;
+        for (int g = 0; g < GC; ++g) acc[g] = 0.f;
         if (works) {
             // pieces of 8 keys; the page numbers and then the values of four pieces are loaded before any is used
             constexpr int PIECES = DEC_KEYS / 8;
@@ -405,7 +418,7 @@ __global__ __launch_bounds__(DEC_KEYS) void decode_values_kernel(
                     const int piece = c0 + u * slices;
                     const int key0 = part * DEC_KEYS + piece * 8;
                     live[u] = piece < PIECES && key0 <= pos && key0 + 7 >= lo;
-                    const long long page = live[u] ? table[key0 / page_size] : 0;
+                    const long long page = live[u] ? page_of[(piece * 8) / page_size] : 0;
                     src[u] = v_cache + ((page * Hkv + kvh) * vd + d) * page_size + key0 % page_size;
                 }
                 bf16x8 vv[4];
@@ -425,8 +438,7 @@ __global__ __launch_bounds__(DEC_KEYS) void decode_values_kernel(
                         // (positions after the last were never written: their weight is 0, but 0 * NaN is not)
                         const float vf = key0 + e <= pos ? (float)vv[u][e] : 0.f;
 #pragma unroll
-                        for (int g = 0; g < DEC_HEADS; ++g)
-                            if (g < Gc) acc[g] = fmaf(wrow[g * DEC_KEYS + e], vf, acc[g]);
+                        for (int g = 0; g < GC; ++g) acc[g] = fmaf(wrow[g * DEC_KEYS + e], vf, acc[g]);     // (g >= Gc: never stored)
                     }
                 }
             }
@@ -434,13 +446,13 @@ __global__ __launch_bounds__(DEC_KEYS) void decode_values_kernel(
         __syncthreads();
         if (works && sl > 0) {
 #pragma unroll
-            for (int g = 0; g < DEC_HEADS; ++g)
+            for (int g = 0; g < GC; ++g)
                 if (g < Gc) w[(g * slices + sl) * vd + d] = acc[g];
         }
         __syncthreads();
         if (works && sl == 0) {
 #pragma unroll
-            for (int g = 0; g < DEC_HEADS; ++g) {
+            for (int g = 0; g < GC; ++g) {
                 if (g < Gc) {
                     float sum = acc[g];
                     for (int s2 = 1; s2 < slices; ++s2) sum += w[(g * slices + s2) * vd + d];
@@ -485,10 +497,15 @@ TUFF_EXPORT int tuff_attention_decode_exact(const void* q, const void* k_cache, 
     if (page_size % 8 != 0 || DEC_KEYS % page_size != 0 || n_parts <= 0 || n_parts > 65535 || Hkv > 65535) return -2;
     if ((log_r1 == nullptr) != (log_r2 == nullptr) || !S || !ml || !po) return -2;
     dim3 grid(n_tokens, Hkv, n_parts), block(DEC_KEYS);
-    hipLaunchKernelGGL(decode_scores_kernel, grid, block, 0, stream, (const bf16_t*)q, (const bf16_t*)k_cache, S, ml, block_table,
-                       max_blocks, req_of_token, positions, H, Hkv, hd, page_size, window, scale, slopes, log_r1, log_r2, n_parts);
-    hipLaunchKernelGGL(decode_values_kernel, grid, block, 0, stream, (const float*)S, (const float*)ml, (const bf16_t*)v_cache, po,
-                       block_table, max_blocks, req_of_token, positions, H, Hkv, vd, page_size, window, sinks, talk, n_parts);
+    // (the loops over a group's heads are unrolled to the power of two that holds them, sixteen at most)
+#define LAUNCH(GC) do { \
+    hipLaunchKernelGGL(decode_scores_kernel<GC>, grid, block, 0, stream, (const bf16_t*)q, (const bf16_t*)k_cache, S, ml, block_table, \
+                       max_blocks, req_of_token, positions, H, Hkv, hd, page_size, window, scale, slopes, log_r1, log_r2, n_parts); \
+    hipLaunchKernelGGL(decode_values_kernel<GC>, grid, block, 0, stream, (const float*)S, (const float*)ml, (const bf16_t*)v_cache, po, \
+                       block_table, max_blocks, req_of_token, positions, H, Hkv, vd, page_size, window, sinks, talk, n_parts); } while (0)
+    const int G = H / Hkv;
+    if (G <= 1) LAUNCH(1); else if (G <= 2) LAUNCH(2); else if (G <= 4) LAUNCH(4); else if (G <= 8) LAUNCH(8); else LAUNCH(16);
+#undef LAUNCH
     dim3 mgrid(n_tokens, H), mblock(WAVE);
     if (out_dt == DT_F32)
         hipLaunchKernelGGL(decode_merge_kernel<float>, mgrid, mblock, 0, stream, (const float*)po, positions, gates, gate_stride,
