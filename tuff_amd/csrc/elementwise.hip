@@ -146,6 +146,22 @@ __global__ void cast_kernel(const TI* __restrict__ in, TO* __restrict__ out, lon
     if (i < n) out[i] = from_f32<TO>(to_f32(in[i]));
 }
 
+// out[i] = in[i] + bias[i % N]: the float32 sums of a product get their bias and are rounded once.
+template <typename TO>
+__global__ void cast_bias_kernel(const float* __restrict__ in, const float* __restrict__ bias, TO* __restrict__ out, long long n, int N) {
+    const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) out[i] = from_f32<TO>(in[i] + bias[i % N]);
+}
+
+TUFF_EXPORT int tuff_cast_bias(const float* in, const float* bias, void* out, int out_dt, long long n, int N, hipStream_t stream) {
+    if (n <= 0) return 0;
+    if (N <= 0 || !bias) return -2;
+    dim3 grid((unsigned)ceil_div_ll(n, 256)), block(256);
+    if (out_dt == DT_BF16) hipLaunchKernelGGL((cast_bias_kernel<bf16_t>), grid, block, 0, stream, in, bias, (bf16_t*)out, n, N);
+    else hipLaunchKernelGGL((cast_bias_kernel<float>), grid, block, 0, stream, in, bias, (float*)out, n, N);
+    return launch_status();
+}
+
 TUFF_EXPORT int tuff_cast(const void* in, int in_dt, void* out, int out_dt, long long n, hipStream_t stream) {
     if (n <= 0) return 0;
     dim3 grid((unsigned)ceil_div_ll(n, 256)), block(256);

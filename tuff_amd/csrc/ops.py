@@ -33,6 +33,7 @@ _SIGNATURES = {
         "tuff_rmsnorm": [_c_void_p, _c_void_p, _c_int, _c_void_p, _c_int, _c_void_p, _c_int, _c_int, _c_float, _c_void_p],
         "tuff_swiglu": [_c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_void_p],
         "tuff_cast": [_c_void_p, _c_int, _c_void_p, _c_int, _c_ll, _c_void_p],
+        "tuff_cast_bias": [_c_void_p, _c_void_p, _c_void_p, _c_int, _c_ll, _c_int, _c_void_p],
         "tuff_fill_u32": [_c_void_p, ctypes.c_uint32, _c_ll, _c_void_p],
         "tuff_scatter_i32": [_c_void_p, _c_int, _c_void_p, _c_int, _c_void_p, _c_int, _c_void_p],
         "tuff_dyt": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_void_p, _c_int, _c_int, _c_void_p],
@@ -109,7 +110,7 @@ _SIGNATURES = {
     },
     "postnorm": {
         "tuff_post_norm_add": [_c_void_p, _c_void_p, _c_void_p, _c_float, _c_float, _c_void_p, _c_void_p, _c_float, _c_void_p,
-                               _c_int, _c_int, _c_int, _c_int, _c_void_p],
+                               _c_int, _c_int, _c_int, _c_int, _c_void_p, _c_void_p],
         "tuff_normed_mean2": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_float, _c_float, _c_void_p, _c_int, _c_int, _c_void_p],
     },
     "hyper": {
@@ -359,9 +360,15 @@ def swiglu(gu: torch.Tensor, act: torch.Tensor) -> None:
         _gpu("gu", gu, act.dtype, (n, 2 * F)), _gpu("act", act), _dt(act), n, F, _stream()), "swiglu")
 
 
-def cast(inp: torch.Tensor, out: torch.Tensor) -> None:
+def cast(inp: torch.Tensor, out: torch.Tensor, bias: Optional[torch.Tensor] = None) -> None:
+    """out = inp in out's type.  bias (float32 [N], inp float32 [rows, N]): out = inp + bias, rounded once."""
     if inp.numel() != out.numel():
         raise KernelError(f"cast: {inp.numel()} elements in, {out.numel()} out")
+    if bias is not None:
+        N = inp.shape[-1]
+        _check(load("elementwise").tuff_cast_bias(_gpu("inp", inp, torch.float32), _gpu("bias", bias, torch.float32, (N,)),
+                                                  _gpu("out", out), _dt(out), inp.numel(), N, _stream()), "cast_bias")
+        return
     _check(load("elementwise").tuff_cast(_gpu("inp", inp), _dt(inp), _gpu("out", out), _dt(out),
                                          inp.numel(), _stream()), "cast")
 
@@ -884,12 +891,14 @@ def head_mix_gate(o, out, *, H, Hkv, vd, talk=None, gates=None) -> None:
 
 # ------------------------------------------------- sublayers normed before they join the stream
 def post_norm_add(x, *, y=None, w=None, eps: float = 0.0, mult: float = 1.0, extra=None, next_w=None, next_eps: float = 0.0,
-                  h_out=None, clear_y: bool = False) -> None:
+                  h_out=None, clear_y: bool = False, y_next=None) -> None:
     """One kernel over the residual stream x (float32 [T, d], in place).  With y float32 [T, d] and w float32 [d]:
     x <- x + mult * y / sqrt(mean(y^2) + eps) * w (y is then cleared, if asked).  With extra float32 [T, d]:
     x <- x + extra.  With next_w float32 [d] and h_out [T, d]: h_out = x / sqrt(mean(x^2) + next_eps) * next_w,
-    from the new x."""
+    from the new x.  y_next float32 [d] (with clear_y): every row of y is left holding y_next instead of zeros, the bias of
+    the product that adds into y next."""
     T, d = x.shape
+    _opt("y_next", y_next, torch.float32, (d,))
     _gpu("x", x, torch.float32, (T, d))
     _opt("y", y, torch.float32, (T, d))
     if y is not None:
@@ -903,7 +912,8 @@ def post_norm_add(x, *, y=None, w=None, eps: float = 0.0, mult: float = 1.0, ext
     _check(load("postnorm").tuff_post_norm_add(
         x.data_ptr(), None if y is None else y.data_ptr(), None if y is None else w.data_ptr(), float(eps), float(mult),
         None if extra is None else extra.data_ptr(), None if next_w is None else next_w.data_ptr(), float(next_eps),
-        None if h_out is None else h_out.data_ptr(), DT_F32 if h_out is None else _dt(h_out), T, d, int(clear_y), _stream()),
+        None if h_out is None else h_out.data_ptr(), DT_F32 if h_out is None else _dt(h_out), T, d, int(clear_y),
+        None if y_next is None else y_next.data_ptr(), _stream()),
         "post_norm_add")
 
 

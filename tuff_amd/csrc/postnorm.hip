@@ -1,7 +1,8 @@
 // Kernels of layers that norm a sublayer's output before it joins the residual stream, all in float32.
 //
 // tuff_post_norm_add, a workgroup a token:
-//     x <- x + mult * y / sqrt(mean(y^2) + eps) * w  [+ extra]        (y is then cleared, if asked)
+//     x <- x + mult * y / sqrt(mean(y^2) + eps) * w  [+ extra]        (y is then cleared, if asked, or set to a row
+//                                                                      y_next: the bias of the product that adds into y next)
 //     h  = x / sqrt(mean(x^2) + eps_next) * w_next                     (if asked: the next sublayer's input)
 // One launch where a norm, a residual sum, another sum and the next norm would be four.  Without y only the
 // sum with `extra` and the next norm run.  The weights come in as float32 with any offset already added.
@@ -23,7 +24,7 @@ template <typename T>
 __global__ __launch_bounds__(PN_THREADS) void post_norm_add_kernel(
     float* __restrict__ x, float* __restrict__ y, const float* __restrict__ w, float eps, float mult,
     const float* __restrict__ extra, const float* __restrict__ w_next, float eps_next, T* __restrict__ h_out,
-    int d, int clear_y) {
+    int d, int clear_y, const float* __restrict__ y_next) {
     __shared__ float scratch[PN_WAVES];
     const long long row = (long long)blockIdx.x * d;
     float* xr = x + row;
@@ -40,7 +41,7 @@ __global__ __launch_bounds__(PN_THREADS) void post_norm_add_kernel(
         float v = xr[c];
         if (y) {
             v = fmaf(y[row + c] * inv, w[c], v);
-            if (clear_y) y[row + c] = 0.f;
+            if (clear_y) y[row + c] = y_next ? y_next[c] : 0.f;
         }
         if (extra) v += extra[row + c];
         if (y || extra) xr[c] = v;
@@ -60,7 +61,7 @@ template <typename T, int EPT>
 __global__ __launch_bounds__(PN_THREADS) void post_norm_add_regs_kernel(
     float* __restrict__ x, float* __restrict__ y, const float* __restrict__ w, float eps, float mult,
     const float* __restrict__ extra, const float* __restrict__ w_next, float eps_next, T* __restrict__ h_out,
-    int d, int clear_y) {
+    int d, int clear_y, const float* __restrict__ y_next) {
     __shared__ float scratch[PN_WAVES];
     const long long row = (long long)blockIdx.x * d;
     float xv[EPT], yv[EPT], wv[EPT], ev[EPT], nv[EPT];
@@ -91,7 +92,7 @@ __global__ __launch_bounds__(PN_THREADS) void post_norm_add_regs_kernel(
         float v = xv[k];
         if (y) {
             v = fmaf(yv[k] * inv, wv[k], v);
-            if (clear_y) y[row + c] = 0.f;
+            if (clear_y) y[row + c] = y_next ? y_next[c] : 0.f;
         }
         if (extra) v += ev[k];
         if (y || extra) x[row + c] = v;
@@ -127,14 +128,14 @@ __global__ __launch_bounds__(PN_THREADS) void normed_mean2_kernel(
 }  // namespace
 
 // x float32 [T][d] in place; y float32 [T][d] or null; w float32 [d] (with y); extra float32 [T][d] or null;
-// w_next float32 [d] and h_out [T][d] of type out_dt, or both null.
+// w_next float32 [d] and h_out [T][d] of type out_dt, or both null; y_next float32 [d] or null (with clear_y).
 TUFF_EXPORT int tuff_post_norm_add(float* x, float* y, const float* w, float eps, float mult, const float* extra,
                                    const float* w_next, float eps_next, void* h_out, int out_dt, int n_tokens, int d,
-                                   int clear_y, hipStream_t stream) {
+                                   int clear_y, const float* y_next, hipStream_t stream) {
     if (n_tokens <= 0) return 0;
     if (d <= 0 || (y && !w) || ((w_next == nullptr) != (h_out == nullptr))) return -2;
     dim3 grid(n_tokens), block(PN_THREADS);
-#define LAUNCH(KERN, T) hipLaunchKernelGGL(KERN, grid, block, 0, stream, x, y, w, eps, mult, extra, w_next, eps_next, (T*)h_out, d, clear_y)
+#define LAUNCH(KERN, T) hipLaunchKernelGGL(KERN, grid, block, 0, stream, x, y, w, eps, mult, extra, w_next, eps_next, (T*)h_out, d, clear_y, y_next)
     if (d <= PN_THREADS * 8) {
         if (out_dt == DT_F32) LAUNCH((post_norm_add_regs_kernel<float, 8>), float); else LAUNCH((post_norm_add_regs_kernel<bf16_t, 8>), bf16_t);
     } else if (d <= PN_THREADS * 32) {

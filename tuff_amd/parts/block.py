@@ -205,18 +205,22 @@ class SandwichBlock(Block):
         self.mixer.forward(carry, ctx, cache, y, write_cache, **kw)
         if self.ffn is None:
             return self._join(x, y, self.after1, next_read, extra)
-        h = self._join(x, y, self.after1, (self.before2.weight_f32, self.before2.eps), None)
+        # (a feed-forward that adds a bias to its output: the kernel that clears y leaves the bias there instead)
+        bias = getattr(self.ffn, "output_bias", None)
+        h = self._join(x, y, self.after1, (self.before2.weight_f32, self.before2.eps), None, y_next=bias)
         kw = {"next_norm": None} if self.ffn.adds_once_through_linear else {}
+        if bias is not None:
+            kw["bias_preloaded"] = True
         self.ffn.forward(h, ctx, y, **kw)
         return self._join(x, y, self.after2, next_read, extra)
 
-    def _join(self, x, y, after, read, extra):
+    def _join(self, x, y, after, read, extra, y_next=None):
         h = None
         kw = {}
         if read is not None:
             h = self.rt.empty(*x.shape)
             kw = dict(next_w=read[0], next_eps=read[1], h_out=h)
-        ops.post_norm_add(x, y=y, w=after.weight_f32, eps=after.eps, mult=self.mult, extra=extra, clear_y=True, **kw)
+        ops.post_norm_add(x, y=y, w=after.weight_f32, eps=after.eps, mult=self.mult, extra=extra, clear_y=True, y_next=y_next, **kw)
         return h
 
 

@@ -155,12 +155,15 @@ class DenseMLP(FeedForward):
         self._make(self.F)
         self._decls = self.up.weight_decls() + self.down.weight_decls()
         if self.has_bias:
-            self._decls.append(WeightDecl(names["up.b"], (self.F,), "normal"))
+            self._decls += [WeightDecl(names["up.b"], (self.F,), "normal"), WeightDecl(names["down.b"], (self.d,), "normal")]
+        #: float32 [d] once bound, or None: what the feed-forward adds to every row of its output.  A block that clears the
+        #: rows its sublayers add into may leave this there instead and say so (forward(bias_preloaded=True))
+        self.output_bias = None
 
     def _make(self, width: int) -> None:
         n = self._names
         self.up = Linear(n["up"], self.d, width)                     # (its bias goes into the activation's kernel)
-        self.down = Linear(n["down"], width, self.d, bias=n["down.b"] if self.has_bias else None)
+        self.down = Linear(n["down"], width, self.d)               # (its bias: output_bias)
         self.width = width
 
     def weight_decls(self):
@@ -185,12 +188,17 @@ class DenseMLP(FeedForward):
         self.up.bind(weights, rt)
         self.down.bind(weights, rt)
         self.up_bias = weights[n["up.b"]].float().contiguous() if self.has_bias else None
+        self.output_bias = weights[n["down.b"]].float().contiguous() if self.has_bias else None
 
-    def forward(self, h, ctx, residual, next_norm=None) -> None:
+    def forward(self, h, ctx, residual, next_norm=None, bias_preloaded: bool = False) -> None:
         u = self.up.forward(h, out_dtype=torch.float32)          # the activation reads the sums as they are, plus the bias
         act = self.rt.empty(u.shape[0], self.width)
         ops.act_rows(u, act, self.activation, bias=self.up_bias)
-        self.down.forward(act, accumulate_into=residual, next_norm=next_norm)
+        if self.output_bias is None or bias_preloaded:
+            self.down.forward(act, accumulate_into=residual, next_norm=next_norm)
+            return
+        self.down.forward(act, accumulate_into=residual)          # (the sum is not final before the bias is in)
+        ops.add_bias(residual, self.output_bias)
 
 
 @FEED_FORWARDS.register("moe")

@@ -188,18 +188,15 @@ class Linear:
         if w.dtype == torch.float32 and want != torch.float32:
             y32 = torch.empty(T, width, dtype=torch.float32, device=dev)
             product(y32)
-            if self.bias is not None:
-                ops.add_bias(y32, self.bias)
             y = torch.empty(T, width, dtype=want, device=dev)
-            ops.cast(y32, y)
+            ops.cast(y32, y, bias=self.bias)
             return y
         if self.bias is not None and want != torch.float32:
             # the bias goes onto the float32 sum, which is then rounded once
             y32 = torch.empty(T, width, dtype=torch.float32, device=dev)
             product(y32)
-            ops.add_bias(y32, self.bias)
             y = torch.empty(T, width, dtype=want, device=dev)
-            ops.cast(y32, y)
+            ops.cast(y32, y, bias=self.bias)            # one kernel: the bias, then the rounding
             return y
         y = torch.empty(T, width, dtype=want, device=dev)
         product(y)
