@@ -8,7 +8,10 @@
 // (scale_input) or y after; act: 0 relu squared, 1 silu, 2 gelu (tanh form).  Gated experts have two first
 // matrices: y = W_down glu(W_gate x, W_up x) with glu(g, u) = act(g) u for the three above, or, act 3, the
 // clamped form g' sigmoid(alpha g') (u' + 1) with g' = min(g, limit), u' = clamp(u, -limit, limit).
-// The router may have a bias: z = W h + b.  A (token, choice) pair is a
+// The router may have a bias: z = W h + b.  A limited choice (sigmoid weights): the choice runs on
+// c = sigmoid(z) + correction instead of z, and only inside the `keep` groups of neighbouring experts (of `groups`
+// equal ones) whose two largest c have the largest sum; the weights are the chosen experts' sigmoid(z), without the
+// correction, times a constant.  A (token, choice) pair is a
 // row of the work arrays; the rows of a token are added into the residual stream in the order of
 // its choices, so the sum does not depend on what else is in the step.
 #include "common.h"
@@ -55,6 +58,53 @@ __device__ void choose(const float* row, int* ids, float* wts, long long t, int 
         for (int s = 0; s < top; ++s) wts[(long long)t * top + s] /= den;
 }
 
+// The limited choice of one token (see the head of the file).  row: its E logits; cs: E floats of scratch.
+// Ties go to the lower index, among groups as among experts.  groups <= 64.
+__device__ void choose_limited(const float* row, float* cs, int* ids, float* wts, long long t, int E, int top,
+                               const float* corr, int groups, int keep, float scale) {
+    for (int e = 0; e < E; ++e) cs[e] = 1.0f / (1.0f + expf(-row[e])) + (corr ? corr[e] : 0.f);
+    const int per = E / groups;
+    unsigned long long kept = ~0ull;
+    if (keep < groups) {
+        kept = 0ull;
+        for (int r = 0; r < keep; ++r) {
+            float best = -INFINITY;
+            int best_g = -1;
+            for (int g = 0; g < groups; ++g) {
+                if ((kept >> g) & 1ull) continue;
+                float m1 = -INFINITY, m2 = -INFINITY;             // the group's two largest
+                for (int e = g * per; e < (g + 1) * per; ++e) {
+                    const float v = cs[e];
+                    if (v > m1) { m2 = m1; m1 = v; } else if (v > m2) m2 = v;
+                }
+                const float score = per > 1 ? m1 + m2 : m1;
+                if (best_g < 0 || score > best) { best = score; best_g = g; }
+            }
+            kept |= 1ull << best_g;
+        }
+    }
+    float last = INFINITY;
+    int last_id = -1;
+    for (int s = 0; s < top; ++s) {
+        float best = -INFINITY;
+        int best_id = -1;
+        for (int e = 0; e < E; ++e) {
+            if (!((kept >> (e / per)) & 1ull)) continue;
+            const float v = cs[e];
+            const bool after = v < last || (v == last && e > last_id);
+            if (after && (best_id < 0 || v > best)) { best = v; best_id = e; }
+        }
+        if (best_id < 0) {                                       // NaN scores: still a valid expert, inside a kept group
+            for (int e = 0; e < E && best_id < 0; ++e)
+                if ((kept >> (e / per)) & 1ull) best_id = e;
+            best = cs[best_id];
+        }
+        ids[(long long)t * top + s] = best_id;
+        wts[(long long)t * top + s] = scale / (1.0f + expf(-row[best_id]));
+        last = best; last_id = best_id;
+    }
+}
+
 __global__ void route_kernel(const float* __restrict__ z, int stride, int* __restrict__ ids, float* __restrict__ wts,
                              int n_tokens, int E, int top, int weight_fn) {
     const int t = blockIdx.x * blockDim.x + threadIdx.x;
@@ -74,11 +124,13 @@ template <typename T, int TB>
 __global__ __launch_bounds__(ROUTER_WAVES * WAVE) void router_kernel(const T* __restrict__ h, const float* __restrict__ W,
                                                                       float* __restrict__ z, int* __restrict__ ids,
                                                                       float* __restrict__ wts, int n_tokens, int d, int N, int E, int top,
-                                                                      int weight_fn, const float* __restrict__ bias) {
+                                                                      int weight_fn, const float* __restrict__ bias,
+                                                                      const float* __restrict__ corr, int groups, int keep, float scale) {
     extern __shared__ __attribute__((aligned(16))) float sm[];
     const int dp = (d + 3) & ~3;
     float* xs = sm;                                        // TB rows of d floats, each padded to a multiple of 4
     float* zs = sm + TB * dp;                              // TB rows of N logits
+    float* cs = zs + TB * N;                               // a limited choice: TB rows of E choice scores
     const long long t0 = (long long)blockIdx.x * TB;
     const int nt = (int)min((long long)TB, n_tokens - t0);
     for (int b = 0; b < TB; ++b)
@@ -118,7 +170,10 @@ __global__ __launch_bounds__(ROUTER_WAVES * WAVE) void router_kernel(const T* __
         }
     }
     __syncthreads();
-    if (threadIdx.x < nt) choose(zs + threadIdx.x * N, ids, wts, t0 + threadIdx.x, E, top, weight_fn);
+    if (threadIdx.x < nt) {
+        if (groups > 0) choose_limited(zs + threadIdx.x * N, cs + threadIdx.x * E, ids, wts, t0 + threadIdx.x, E, top, corr, groups, keep, scale);
+        else choose(zs + threadIdx.x * N, ids, wts, t0 + threadIdx.x, E, top, weight_fn);
+    }
 }
 
 constexpr int ROWS_WG = 16;          // output rows a workgroup of four waves computes
@@ -344,17 +399,21 @@ TUFF_EXPORT int tuff_moe_experts(const void* h, const void* w_up, const void* w_
 }
 
 // z float32 [T][N], the first E columns the experts' logits; ids, wts [T][top].  W float32 [N][d]; h [T][d] of type dt.
-// bias float32 [E] or null: added to the experts' logits before the choice.
+// bias float32 [E] or null: added to the experts' logits before the choice.  groups > 0: the limited choice (weight_fn 0),
+// with corr float32 [E] or null, `keep` of `groups` groups and the weights times `scale`; groups 0: the plain choice.
 TUFF_EXPORT int tuff_moe_router(const void* h, int dt, const float* W, float* z, int* ids, float* wts, int n_tokens, int d,
-                                int N, int E, int top, int weight_fn, const float* bias, hipStream_t stream) {
+                                int N, int E, int top, int weight_fn, const float* bias, const float* corr, int groups, int keep,
+                                float scale, hipStream_t stream) {
     if (n_tokens <= 0) return 0;
-    if (top < 1 || top > E || N < E || (long long)(d + 4 + N) * 4 > 65536) return -2;
+    const int extra = groups > 0 ? E : 0;
+    if (top < 1 || top > E || N < E || (long long)(d + 4 + N + extra) * 4 > 65536) return -2;
+    if (groups > 0 && (weight_fn != 0 || groups > 64 || E % groups || keep < 1 || keep > groups || top > keep * (E / groups))) return -2;
     // long steps: four tokens a workgroup where that fits the LDS (the rows of W are then read a quarter as often)
-    const bool four = n_tokens >= 1024 && (long long)(d + 4 + N) * 16 <= 65536;
+    const bool four = n_tokens >= 1024 && (long long)(d + 4 + N + extra) * 16 <= 65536;
     const int TB = four ? 4 : 1;
-    const size_t lds = (size_t)TB * (((d + 3) & ~3) + N) * sizeof(float);
+    const size_t lds = (size_t)TB * (((d + 3) & ~3) + N + extra) * sizeof(float);
     const dim3 grid((unsigned)ceil_div(n_tokens, TB)), block(ROUTER_WAVES * WAVE);
-#define LAUNCH(T, B) hipLaunchKernelGGL((router_kernel<T, B>), grid, block, lds, stream, (const T*)h, W, z, ids, wts, n_tokens, d, N, E, top, weight_fn, bias)
+#define LAUNCH(T, B) hipLaunchKernelGGL((router_kernel<T, B>), grid, block, lds, stream, (const T*)h, W, z, ids, wts, n_tokens, d, N, E, top, weight_fn, bias, corr, groups, keep, scale)
     if (dt == DT_F32) { if (four) LAUNCH(float, 4); else LAUNCH(float, 1); }
     else { if (four) LAUNCH(bf16_t, 4); else LAUNCH(bf16_t, 1); }
 #undef LAUNCH

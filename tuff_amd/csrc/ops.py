@@ -45,22 +45,25 @@ _SIGNATURES = {
         "tuff_shift_mix": [_c_void_p, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p,
                            _c_int, _c_int, _c_int, _c_void_p],
         "tuff_shift_state": [_c_void_p, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_void_p],
-        "tuff_conv_act": [_c_void_p, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p,
-                          _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p],
+        "tuff_conv_act": [_c_void_p, _c_int, _c_ll, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_void_p, _c_void_p, _c_void_p,
+                          _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p],
         "tuff_wkv_scan": [_c_void_p, _c_void_p, _c_void_p, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p,
                           _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_void_p],
-        "tuff_delta_scan": [_c_void_p, _c_void_p, _c_void_p, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p,
-                            _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int,
+        "tuff_delta_scan": [_c_void_p, _c_void_p, _c_void_p, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_ll,
+                            _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int,
                             _c_int, _c_int, _c_int, _c_ll, _c_ll, _c_void_p],
-        "tuff_head_norm_gate": [_c_void_p, _c_void_p, _c_int, _c_void_p, _c_int, _c_int, _c_int, _c_void_p, _c_int, _c_int, _c_int,
-                                _c_float, _c_void_p],
+        "tuff_head_norm_gate": [_c_void_p, _c_void_p, _c_int, _c_void_p, _c_ll, _c_int, _c_int, _c_int, _c_int, _c_void_p, _c_int, _c_int,
+                                _c_int, _c_float, _c_void_p],
+        "tuff_ssd_scan": [_c_void_p, _c_int, _c_ll, _c_void_p, _c_ll, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p,
+                          _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int,
+                          _c_int, _c_void_p],
         "tuff_forget_scan": [_c_void_p, _c_int, _c_ll, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p,
                              _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p],
     },
     "moe": {
         "tuff_moe_route": [_c_void_p, _c_int, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_void_p],
         "tuff_moe_router": [_c_void_p, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int,
-                            _c_int, _c_void_p, _c_void_p],
+                            _c_int, _c_void_p, _c_void_p, _c_int, _c_int, _c_float, _c_void_p],
         "tuff_moe_grouped_tile_rows": [_c_ll, _c_int],
         "tuff_moe_grouped_wide_from": [_c_int],
         "tuff_moe_grouped_tiled_from": [_c_int],
@@ -112,6 +115,8 @@ _SIGNATURES = {
         "tuff_post_norm_add": [_c_void_p, _c_void_p, _c_void_p, _c_float, _c_float, _c_void_p, _c_void_p, _c_float, _c_void_p,
                                _c_int, _c_int, _c_int, _c_int, _c_void_p, _c_void_p],
         "tuff_normed_mean2": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_float, _c_float, _c_void_p, _c_int, _c_int, _c_void_p],
+        "tuff_scale_add_layer_norm": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_float, _c_void_p, _c_int, _c_void_p, _c_int, _c_int,
+                                      _c_int, _c_void_p],
     },
     "hyper": {
         "tuff_hc_step": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_void_p,
@@ -917,6 +922,32 @@ def post_norm_add(x, *, y=None, w=None, eps: float = 0.0, mult: float = 1.0, ext
         "post_norm_add")
 
 
+def scale_add_layer_norm(x, *, y=None, ls=None, next_w=None, eps: float = 0.0, h_out=None, rows=None, clear_y: bool = False) -> None:
+    """One kernel over the residual stream x (float32 [T, d], in place).  With y float32 [T, d] and ls float32 [d]:
+    x <- x + ls * y (y is then cleared, if asked).  With next_w float32 [d] and h_out: h_out = (x - mean) /
+    sqrt(mean((x - mean)^2) + eps) * next_w from the new x, a layer norm with a weight and no bias.  rows (int32 [n],
+    only without y): h_out [n, d] holds the norm of those rows of x, in that order."""
+    T, d = x.shape
+    _gpu("x", x, torch.float32, (T, d))
+    if (y is None) != (ls is None):
+        raise KernelError("scale_add_layer_norm: y and ls go together")
+    if (next_w is None) != (h_out is None):
+        raise KernelError("scale_add_layer_norm: next_w and h_out go together")
+    if rows is not None and y is not None:
+        raise KernelError("scale_add_layer_norm: chosen rows go with the norm alone")
+    _opt("y", y, torch.float32, (T, d))
+    _opt("ls", ls, torch.float32, (d,))
+    n = T if rows is None else rows.shape[0]
+    _opt("rows", rows, torch.int32, (n,))
+    if next_w is not None:
+        _gpu("next_w", next_w, torch.float32, (d,))
+        _gpu("h_out", h_out, shape=(n, d))
+    p = lambda t: None if t is None else t.data_ptr()
+    _check(load("postnorm").tuff_scale_add_layer_norm(
+        x.data_ptr(), p(y), p(ls), p(next_w), float(eps), p(h_out), DT_F32 if h_out is None else _dt(h_out), p(rows), n, d,
+        int(bool(clear_y)), _stream()), "scale_add_layer_norm")
+
+
 def normed_mean2(a, wa, b, wb, out, *, eps: float, coef: float = 0.5) -> None:
     """out <- out + coef * (a / sqrt(mean(a^2) + eps) * wa + b / sqrt(mean(b^2) + eps) * wb); a, b, out float32
     [T, d]; wa, wb float32 [d]."""
@@ -1485,10 +1516,25 @@ def shift_state(h, prev_state, *, q_start, q_len, state_slot) -> None:
 CONV_ACT_MAX_TAPS = 17
 
 
-def conv_act(x, taps, state, out, *, req_of_token, q_start, state_slot, q_len=None, activation: Optional[str] = "silu") -> None:
-    """out[t, c] = activation(sum_j taps[c, j] x[t - (K - 1) + j, c]) along each request; rows before the
+def _rows_view(name: str, t: torch.Tensor, width: Optional[int] = None) -> int:
+    """Checks a [T, width] tensor on the GPU whose rows may be a column range of a wider tensor (unit column
+    stride, any row stride of at least the width); returns the row stride in elements."""
+    if not isinstance(t, torch.Tensor) or not t.is_cuda:
+        raise KernelError(f"{name}: expected a tensor on the GPU")
+    if t.dim() != 2 or (width is not None and t.shape[1] != width) or (t.shape[1] > 1 and t.stride(1) != 1):
+        raise KernelError(f"{name}: expected [tokens, {width}] with unit column stride, got {tuple(t.shape)} stride {t.stride()}")
+    ld = t.stride(0) if t.shape[0] > 1 else max(t.stride(0), t.shape[1])
+    if ld < t.shape[1]:
+        raise KernelError(f"{name}: rows overlap (stride {t.stride()})")
+    return ld
+
+
+def conv_act(x, taps, state, out, *, req_of_token, q_start, state_slot, q_len=None, activation: Optional[str] = "silu",
+             bias=None) -> None:
+    """out[t, c] = activation(sum_j taps[c, j] x[t - (K - 1) + j, c] + bias[c]) along each request; rows before the
     step's first come from state[slot] (float32 [slots, K - 1, C]; None with one tap).  With q_len the state
-    is then rewritten with the last K - 1 inputs; without, it is only read."""
+    is then rewritten with the last K - 1 inputs; without, it is only read.  x may be a column range of a wider
+    tensor, and float32 where out is bfloat16 (a product's sums as they are); bias float32 [C] or None."""
     T, C = x.shape
     K = taps.shape[1]
     R = q_start.shape[0]
@@ -1498,9 +1544,13 @@ def conv_act(x, taps, state, out, *, req_of_token, q_start, state_slot, q_len=No
         raise KernelError(f"conv_act: 1 to {CONV_ACT_MAX_TAPS} taps, got {K}")
     if K > 1:
         _gpu("state", state, torch.float32, (None, K - 1, C))
+    ldx = _rows_view("x", x)
+    if x.dtype != out.dtype and x.dtype != torch.float32:
+        raise KernelError(f"conv_act: input {x.dtype} with output {out.dtype}")
     _check(load("recurrent").tuff_conv_act(
-        _gpu("x", x), _dt(x), _gpu("taps", taps, torch.float32, (C, K)), None if K == 1 else state.data_ptr(),
-        _gpu("out", out, x.dtype, (T, C)), _gpu("req_of_token", req_of_token, torch.int32, (T,)),
+        x.data_ptr(), _dt(x), ldx, _gpu("taps", taps, torch.float32, (C, K)), _opt("bias", bias, torch.float32, (C,)),
+        None if K == 1 else state.data_ptr(),
+        _gpu("out", out, shape=(T, C)), _dt(out), _gpu("req_of_token", req_of_token, torch.int32, (T,)),
         _gpu("q_start", q_start, torch.int32, (R,)), _opt("q_len", q_len, torch.int32, (R,)),
         _gpu("state_slot", state_slot, torch.int32, (R,)), T, R, C, K, 1 if activation == "silu" else 0, _stream()), "conv_act")
 
@@ -1527,12 +1577,13 @@ def wkv_scan(r, k, v, lw, w0, u, state, out, *, q_start, q_len, state_slot, H, D
         _gpu("state_slot", state_slot, torch.int32, (R,)), T, R, H, D, _stream()), "wkv_scan")
 
 
-def delta_scan(q, k, v, a, dt_bias, A_log, b, state, out, *, q_start, q_len, state_slot, H, Hk, D, Dv) -> None:
+def delta_scan(q, k, v, a, dt_bias, A_log, b, state, out, *, q_start, q_len, state_slot, H, Hk, D, Dv, per_head: bool = False) -> None:
     """The gated delta rule over each request's tokens of the step, from and to state[slot] (float32
     [slots, H, D, Dv]): S = g S; e = beta (v - S^T k); S = S + k e^T; o = S^T q, with q and k made unit
     vectors per head (q also times D^-1/2), g = exp(-exp(A_log) softplus(a + dt_bias)), beta = sigmoid(b).
-    q, k [T, Hk * D]; v [T, H * Dv]; a float32 [T, H * D] (overwritten with the decays); b float32 [T, H]; out
-    float32 [T, H * Dv]."""
+    q, k [T, Hk * D]; v [T, H * Dv]; a float32 [T, H * D] (overwritten with the decays) and dt_bias [H * D]; b float32
+    [T, H]; out float32 [T, H * Dv].  per_head: one decay per head, a float32 [T, H] and dt_bias [H] (a and b may then
+    be column ranges of one wider tensor, with one row stride)."""
     T = q.shape[0]
     R = q_start.shape[0]
     dt = q.dtype
@@ -1546,14 +1597,52 @@ def delta_scan(q, k, v, a, dt_bias, A_log, b, state, out, *, q_start, q_len, sta
     if D > SCAN_MAX_DIM or Hk < 1 or H % Hk:
         raise KernelError(f"delta_scan: key size {D} (at most {SCAN_MAX_DIM}) / heads {H}:{Hk} not supported")
     work = torch.empty(2, T, H * D, dtype=torch.float32, device=q.device)       # q and k as unit vectors
+    if per_head:
+        ld_small = _rows_view("b", b, H)
+        if a.dtype != torch.float32 or b.dtype != torch.float32 or _rows_view("a", a, H) != ld_small:
+            raise KernelError("delta_scan: a and b must be float32 [tokens, heads] with one row stride")
+        decays = torch.empty(T, H * D, dtype=torch.float32, device=q.device)
+        a_head, a_ptr = a.data_ptr(), decays.data_ptr()
+        _gpu("dt_bias", dt_bias, torch.float32, (H,))
+    else:
+        ld_small, a_head = H, None
+        a_ptr = _gpu("a", a, torch.float32, (T, H * D))
+        _gpu("dt_bias", dt_bias, torch.float32, (H * D,))
+        _gpu("b", b, torch.float32, (T, H))
     _check(load("recurrent").tuff_delta_scan(
         q.data_ptr(), k.data_ptr(), v.data_ptr(), _dt(q),
-        _gpu("a", a, torch.float32, (T, H * D)), _gpu("dt_bias", dt_bias, torch.float32, (H * D,)),
-        _gpu("A_log", A_log, torch.float32, (H,)), _gpu("b", b, torch.float32, (T, H)),
+        a_ptr, dt_bias.data_ptr(), _gpu("A_log", A_log, torch.float32, (H,)), b.data_ptr(), a_head, ld_small,
         work[0].data_ptr(), work[1].data_ptr(), torch.empty(T, H, dtype=torch.float32, device=q.device).data_ptr(),
         _gpu("state", state, torch.float32, (None, H, D, Dv)), _gpu("out", out, torch.float32, (T, H * Dv)),
         _gpu("q_start", q_start, torch.int32, (R,)), _gpu("q_len", q_len, torch.int32, (R,)),
         _gpu("state_slot", state_slot, torch.int32, (R,)), T, R, H, Hk, D, Dv, ld, ldv, _stream()), "delta_scan")
+
+
+def ssd_scan(xbc, dt_raw, dt_bias, A_log, D_skip, state, out, *, q_start, q_len, state_slot, H, G, N, P) -> None:
+    """The state-space recurrence with a scalar decay per head over each request's tokens of the step, from and to
+    state[slot] (float32 [slots, H, N, P]): with dt = softplus(dt_raw + dt_bias) per head,
+    S = exp(-exp(A_log) dt) S + dt B x^T;  y = S^T C + D_skip x  (the read sees the token's own write).
+    xbc [T, H P + 2 G N]: a token's x, B and C side by side (after their convolution), head h reading B and C of
+    group h // (H / G); dt_raw float32 [T, H] (it may be a column range of a wider tensor); dt_bias, A_log, D_skip
+    float32 [H]; out float32 [T, H * P]."""
+    T = xbc.shape[0]
+    R = q_start.shape[0]
+    if N > SCAN_MAX_DIM:
+        raise KernelError(f"ssd_scan: state size {N} above {SCAN_MAX_DIM}")
+    if G < 1 or H % G:
+        raise KernelError(f"ssd_scan: {H} heads in {G} groups")
+    ld = _rows_view("xbc", xbc, H * P + 2 * G * N)
+    ld_dt = _rows_view("dt_raw", dt_raw, H)
+    if dt_raw.dtype != torch.float32:
+        raise KernelError("ssd_scan: dt_raw must be float32")
+    work = torch.empty(3, T, H * N, dtype=torch.float32, device=xbc.device)     # queries, keys, decays
+    _check(load("recurrent").tuff_ssd_scan(
+        xbc.data_ptr(), _dt(xbc), ld, dt_raw.data_ptr(), ld_dt, _gpu("dt_bias", dt_bias, torch.float32, (H,)),
+        _gpu("A_log", A_log, torch.float32, (H,)), _gpu("D_skip", D_skip, torch.float32, (H,)),
+        work[0].data_ptr(), work[1].data_ptr(), work[2].data_ptr(), torch.empty(T, H, dtype=torch.float32, device=xbc.device).data_ptr(),
+        _gpu("state", state, torch.float32, (None, H, N, P)), _gpu("out", out, torch.float32, (T, H * P)),
+        _gpu("q_start", q_start, torch.int32, (R,)), _gpu("q_len", q_len, torch.int32, (R,)),
+        _gpu("state_slot", state_slot, torch.int32, (R,)), T, R, H, G, N, P, _stream()), "ssd_scan")
 
 
 def forget_scan(x, bias, lower, state, out, *, q_start, q_len, state_slot, H, D, Dv) -> None:
@@ -1574,16 +1663,19 @@ def forget_scan(x, bias, lower, state, out, *, q_start, q_len, state_slot, H, D,
         _gpu("state_slot", state_slot, torch.int32, (R,)), T, R, H, D, Dv, _stream()), "forget_scan")
 
 
-def head_norm_gate(o, w, gate, out, *, H, Dv, eps, per_head_weight: bool, gate_activation: Optional[str]) -> None:
+def head_norm_gate(o, w, gate, out, *, H, Dv, eps, per_head_weight: bool, gate_activation: Optional[str],
+                   gate_first: bool = False) -> None:
     """out[t, h] = o[t, h] / sqrt(mean(o[t, h]^2) + eps) * w * f(gate[t, h]); o float32 [T, H * Dv]; w float32
     [H * Dv] (per_head_weight) or [Dv] (shared by the heads); out [T, H * Dv] of the compute type, gate of that
-    type or float32, or None for no gate."""
+    type or float32 (it may be a column range of a wider tensor), or None for no gate.  gate_first: the gate comes
+    before the norm, out = u / sqrt(mean(u^2) + eps) * w with u = o f(gate)."""
     T = o.shape[0]
+    gate_ld = 0 if gate is None else _rows_view("gate", gate, H * Dv)
     _check(load("recurrent").tuff_head_norm_gate(
         _gpu("o", o, torch.float32, (T, H * Dv)), _gpu("w", w, torch.float32, (H * Dv if per_head_weight else Dv,)),
-        Dv if per_head_weight else 0, _opt("gate", gate, shape=(T, H * Dv)), _dt(out if gate is None else gate), _dt(out),
-        {None: 0, "silu": 1, "sigmoid": 2}[gate_activation], _gpu("out", out, shape=(T, H * Dv)), T, H, Dv, float(eps), _stream()),
-        "head_norm_gate")
+        Dv if per_head_weight else 0, None if gate is None else gate.data_ptr(), gate_ld, _dt(out if gate is None else gate), _dt(out),
+        {None: 0, "silu": 1, "sigmoid": 2}[gate_activation], int(bool(gate_first)), _gpu("out", out, shape=(T, H * Dv)), T, H, Dv,
+        float(eps), _stream()), "head_norm_gate")
 
 
 # ------------------------------------------------------------------ mixture of experts
@@ -1602,17 +1694,24 @@ def moe_route(z, ids, wts, *, E, top, weights: str = "sigmoid") -> None:
 ROUTER_MAX_FLOATS = 16380          # hidden size + logits a token: what the router kernel keeps in LDS
 
 
-def moe_router(h, w, z, ids, wts, *, E, top, weights: str = "sigmoid", bias=None) -> None:
+def moe_router(h, w, z, ids, wts, *, E, top, weights: str = "sigmoid", bias=None, correction=None, groups: int = 0,
+               keep: int = 0, scale: float = 1.0) -> None:
     """z = h @ w.T in float32 (h [T, d] of the compute type, w float32 [N, d], z float32 [T, N]) and, of its first
-    E columns, the choice as moe_route makes it, in one kernel.  bias: float32 [E], added to the experts' logits."""
+    E columns, the choice as moe_route makes it, in one kernel.  bias: float32 [E], added to the experts' logits.
+    groups > 0 (sigmoid weights): a limited choice.  It runs on sigmoid(z) + correction (float32 [E] or None) and only
+    inside the `keep` groups, of `groups` equal groups of neighbouring experts, whose two largest such scores have the
+    largest sum; the weights are sigmoid(z) of the chosen, without the correction, times `scale`."""
     T, d = h.shape
     N = w.shape[0]
-    if d + N > ROUTER_MAX_FLOATS:
+    if d + N + (E if groups else 0) > ROUTER_MAX_FLOATS:
         raise KernelError(f"moe_router: hidden size {d} + {N} logits above {ROUTER_MAX_FLOATS}")
+    if groups and (weights != "sigmoid" or groups > 64 or E % groups or not 1 <= keep <= groups or top > keep * (E // groups)):
+        raise KernelError(f"moe_router: a limited choice of {top} among {keep} of {groups} groups of {E} experts is not possible")
     _check(load("moe").tuff_moe_router(_gpu("h", h), _dt(h), _gpu("w", w, torch.float32, (N, d)), _gpu("z", z, torch.float32, (T, N)),
                                        _gpu("ids", ids, torch.int32, (T, top)), _gpu("wts", wts, torch.float32, (T, top)),
                                        T, d, N, E, top, {"sigmoid": 0, "softmax": 1}[weights],
-                                       _opt("bias", bias, torch.float32, (E,)), _stream()), "moe_router")
+                                       _opt("bias", bias, torch.float32, (E,)), _opt("correction", correction, torch.float32, (E,)),
+                                       int(groups), int(keep), float(scale), _stream()), "moe_router")
 
 
 def tile_experts(ws) -> torch.Tensor:

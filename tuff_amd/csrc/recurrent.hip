@@ -1,7 +1,8 @@
 // Kernels of mixers that carry a fixed-size state from token to token: the blend of a token's input
 // with the one before it (token shift), a short causal convolution per channel with an activation,
-// and three matrix-state recurrences, a decaying outer-product memory with a bonus for the current
-// token ("wkv"), a gated delta rule, and a memory whose forget gate also sets the write strength.  States are float32 and live in a slot per request; a step
+// and four matrix-state recurrences, a decaying outer-product memory with a bonus for the current
+// token ("wkv"), a gated delta rule (a decay per key channel or one per head), a memory whose forget gate also
+// sets the write strength, and the state-space recurrence with a scalar decay per head ("ssd").  States are float32 and live in a slot per request; a step
 // brings each request's next tokens (one decoded token or a portion of a prompt of any length),
 // tokens flat and ordered by request, and every kernel continues from the slot and leaves it ready
 // for the next step.  The recurrences run token by token in one fixed order of operations, so a
@@ -58,32 +59,33 @@ __global__ void shift_state_kernel(const T* __restrict__ h, float* __restrict__ 
 }
 
 // --------------------------------------------------------------- short causal convolution
-// y[t][c] = act(sum_j taps[c][j] x[t - (K-1) + j][c]); inputs before the step's first token come from
-// the request's state [K-1][C] (zeros for a new request).  act: 0 none, 1 silu.
+// y[t][c] = act(sum_j taps[c][j] x[t - (K-1) + j][c] + bias[c]); inputs before the step's first token come from
+// the request's state [K-1][C] (zeros for a new request).  act: 0 none, 1 silu.  The rows of x lie ldx elements
+// apart (they may be a column range of a wider projected row) and may be of another type than y's.
 constexpr int MAX_TAPS = 17;
 
-template <typename T>
-__global__ void conv_act_kernel(const T* __restrict__ x, const float* __restrict__ taps, const float* __restrict__ state,
-                                T* __restrict__ y, const int* __restrict__ req_of_token, const int* __restrict__ q_start,
-                                const int* __restrict__ state_slot, int C, int K, int act) {
+template <typename T, typename TY>
+__global__ void conv_act_kernel(const T* __restrict__ x, long long ldx, const float* __restrict__ taps, const float* __restrict__ bias,
+                                const float* __restrict__ state, TY* __restrict__ y, const int* __restrict__ req_of_token,
+                                const int* __restrict__ q_start, const int* __restrict__ state_slot, int C, int K, int act) {
     const int t = blockIdx.x;
     const int r = req_of_token[t];
     const int i = t - q_start[r];                     // index within the step's portion
     const float* st = state + (long long)state_slot[r] * (K - 1) * C;
     for (int c = blockIdx.y * blockDim.x + threadIdx.x; c < C; c += gridDim.y * blockDim.x) {
-        float acc = 0.f;
+        float acc = bias ? bias[c] : 0.f;
         for (int j = 0; j < K; ++j) {
             const int li = i - (K - 1) + j;
-            const float v = li >= 0 ? to_f32(x[(long long)(t - (K - 1) + j) * C + c]) : st[(long long)(i + j) * C + c];
+            const float v = li >= 0 ? to_f32(x[(long long)(t - (K - 1) + j) * ldx + c]) : st[(long long)(i + j) * C + c];
             acc = fmaf(taps[(long long)c * K + j], v, acc);
         }
-        y[(long long)t * C + c] = from_f32<T>(act == 1 ? siluf_(acc) : acc);
+        y[(long long)t * C + c] = from_f32<TY>(act == 1 ? siluf_(acc) : acc);
     }
 }
 
 // the state after the step: the last K-1 inputs, from the step's rows and, for a short portion, the old state
 template <typename T>
-__global__ void conv_state_kernel(const T* __restrict__ x, float* __restrict__ state, const int* __restrict__ q_start,
+__global__ void conv_state_kernel(const T* __restrict__ x, long long ldx, float* __restrict__ state, const int* __restrict__ q_start,
                                   const int* __restrict__ q_len, const int* __restrict__ state_slot, int C, int K) {
     const int r = blockIdx.x;
     const int n = q_len[r];
@@ -96,7 +98,7 @@ __global__ void conv_state_kernel(const T* __restrict__ x, float* __restrict__ s
         for (int m = 0; m < MAX_TAPS - 1; ++m) {
             if (m < K - 1) {
                 const int li = n - (K - 1) + m;
-                keep[m] = li >= 0 ? to_f32(x[(long long)(t0 + li) * C + c]) : st[(long long)(m + n) * C + c];
+                keep[m] = li >= 0 ? to_f32(x[(long long)(t0 + li) * ldx + c]) : st[(long long)(m + n) * C + c];
             }
         }
 #pragma unroll
@@ -128,7 +130,10 @@ struct PrepArgs {
     float* decay;                   // in: lw or a [T][H*D]; out, in place: w or g
     const float* decay_bias;        // [H*D]: w0 or dt_bias
     const float* per_head;          // wkv: u [H][D];  delta: A_log [H]
-    const float* beta_in;           // delta: b [T][H]
+    const float* beta_in;           // delta: b, a token's H values ld_small apart
+    const float* head_decay_in;     // delta with one decay per head: a, a token's H values ld_small apart (decay_bias is
+                                    // then [H]); null: the decay's inputs are a value per key channel, in `decay`
+    long long ld_small;
     float *qn, *kn;                 // delta, out: unit vectors [T][H][D]
     float* scalar;                  // out [T][H]: bonus (wkv) or beta (delta)
     int H, Ha, D;
@@ -154,12 +159,14 @@ __global__ __launch_bounds__(WAVE) void scan_prep_kernel(PrepArgs p) {
         qq = wave_sum(qq); kk = wave_sum(kk);
         const float qn = (1.0f / sqrtf((float)D)) / sqrtf(qq + 1e-6f), kn = 1.0f / sqrtf(kk + 1e-6f);
         const float neg_rate = -expf(p.per_head[head]);
+        const float g_head = p.head_decay_in
+            ? expf(neg_rate * softplusf_(p.head_decay_in[t * p.ld_small + head] + p.decay_bias[head])) : 0.f;
         for (int i = lane; i < D; i += WAVE) {
             p.qn[(t * H + head) * D + i] = to_f32(pa[i]) * qn;
             p.kn[(t * H + head) * D + i] = to_f32(pk[i]) * kn;
-            dec[i] = expf(neg_rate * softplusf_(dec[i] + p.decay_bias[head * D + i]));
+            dec[i] = p.head_decay_in ? g_head : expf(neg_rate * softplusf_(dec[i] + p.decay_bias[head * D + i]));
         }
-        if (lane == 0) p.scalar[t * H + head] = sigmoidf_(p.beta_in[t * H + head]);
+        if (lane == 0) p.scalar[t * H + head] = sigmoidf_(p.beta_in[t * p.ld_small + head]);
     } else {
         float bonus = 0.f;
         for (int i = lane; i < D; i += WAVE) {
@@ -183,6 +190,32 @@ __global__ void forget_prep_kernel(const T* __restrict__ x, long long ld, const 
         qn[t * HD + c] = siluf_(to_f32(row[c]));
         f[t * HD + c] = lo + (1.0f - lo) * sigmoidf_(to_f32(row[HD + c]) + (bias ? bias[c] : 0.f));
     }
+}
+
+// What enters the state-space recurrence of head h (group g = h / (H / G)) at token t, all float32:
+// dt = softplus(dt_raw + dt_bias_h), decay = exp(-exp(A_log_h) dt) (the same for all N state channels),
+// key = dt B[t][g], query = C[t][g], and the head's D as the bonus on the token's own input.
+// bc: a token's convolved rows [.. | B (G*N) | C (G*N)] of type T, ldbc apart, B from column b_off.
+// dt_raw float32, a token's H values ld_dt apart.
+template <typename T>
+__global__ __launch_bounds__(WAVE) void ssd_prep_kernel(const T* __restrict__ bc, long long ldbc, int b_off, const float* __restrict__ dt_raw,
+                                                        long long ld_dt, const float* __restrict__ dt_bias, const float* __restrict__ A_log,
+                                                        const float* __restrict__ Dh, float* __restrict__ qn, float* __restrict__ kn,
+                                                        float* __restrict__ decay, float* __restrict__ scalar, int H, int G, int N) {
+    const long long t = blockIdx.x;
+    const int head = blockIdx.y, lane = threadIdx.x;
+    const int g = head / (H / G);
+    const float dt = softplusf_(dt_raw[t * ld_dt + head] + dt_bias[head]);
+    const float dec = expf(-expf(A_log[head]) * dt);
+    const T* pb = bc + t * ldbc + b_off + (long long)g * N;
+    const T* pc = pb + (long long)G * N;
+    const long long o = (t * H + head) * N;
+    for (int i = lane; i < N; i += WAVE) {
+        kn[o + i] = dt * to_f32(pb[i]);
+        qn[o + i] = to_f32(pc[i]);
+        decay[o + i] = dec;
+    }
+    if (lane == 0) scalar[t * H + head] = Dh[head];
 }
 
 struct ScanArgs {
@@ -217,7 +250,8 @@ __device__ __forceinline__ float group_sum(float v) {
 
 // TA: type of a and k (the compute type for wkv's r and k, float for the delta rule's unit vectors); T: type of v.
 // FORGET: a holds silu(q) in float32, the decay is the forget gate f and the key is 1 - f (k and scalar are not used).
-template <typename TA, typename T, int NI16, int SPLIT, bool DELTA, bool FORGET = false>
+// SSD: S_ij <- w_i S_ij + k_i v_j, then o_j = sum_i a_i S_ij + scalar v_j (the read sees the token's own write).
+template <typename TA, typename T, int NI16, int SPLIT, bool DELTA, bool FORGET = false, bool SSD = false>
 __global__ __launch_bounds__(WAVE) void scan_kernel(ScanArgs p) {
     constexpr int RP = NI16 * 4;                       // rows of the state's column a lane keeps
     constexpr int DP = RP * SPLIT;                     // key channels, padded
@@ -315,7 +349,7 @@ __global__ __launch_bounds__(WAVE) void scan_kernel(ScanArgs p) {
                 const f32x4 r4 = *(const f32x4*)&sa[tt][row0 + g4 * 4];
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
-                    if (FORGET) {
+                    if (FORGET || SSD) {
                         s[g4 * 4 + e] = fmaf(w4[e], s[g4 * 4 + e], k4[e] * vt);
                         o4[e] = fmaf(r4[e], s[g4 * 4 + e], o4[e]);
                     } else {
@@ -375,25 +409,36 @@ __global__ __launch_bounds__(WAVE) void scan_kernel(ScanArgs p) {
 // ---------------------------------------------------------- per-head unit norm, weight and gate
 // y[t][h][j] = o[t][h][j] / sqrt(mean_j o^2 + eps) * w[(h * w_stride) + j] * f(gate[t][h][j]);
 // f: 0 identity, 1 silu, 2 sigmoid; without a gate the factor is 1.  A wave per (token, head).
+// gate_first: the gate comes before the norm, y = u / sqrt(mean_j u^2 + eps) * w with u = o f(gate).
+// A token's gates lie gate_ld elements apart (they may be a column range of a wider projected row).
 template <typename TG, typename T>
 __global__ __launch_bounds__(WAVE) void head_norm_gate_kernel(const float* __restrict__ o, const float* __restrict__ w, int w_stride,
-                                                              const TG* __restrict__ gate, int gate_fn, T* __restrict__ y,
-                                                              int H, int Dv, float eps) {
+                                                              const TG* __restrict__ gate, long long gate_ld, int gate_fn, int gate_first,
+                                                              T* __restrict__ y, int H, int Dv, float eps) {
     const long long row = (long long)blockIdx.x * H + blockIdx.y;
     const float* src = o + row * Dv;
+    const TG* gr = gate ? gate + (long long)blockIdx.x * gate_ld + (long long)blockIdx.y * Dv : nullptr;
+    auto gate_of = [&](int j) {
+        float g = gr ? to_f32(gr[j]) : 1.f;
+        if (gate_fn == 1) g = siluf_(g);
+        else if (gate_fn == 2) g = sigmoidf_(g);
+        return g;
+    };
     float ss = 0.f;
-    for (int j = threadIdx.x; j < Dv; j += WAVE) ss = fmaf(src[j], src[j], ss);
+    for (int j = threadIdx.x; j < Dv; j += WAVE) {
+        const float u = gate_first ? src[j] * gate_of(j) : src[j];
+        ss = fmaf(u, u, ss);
+    }
     ss = wave_sum(ss);
     const float inv = 1.0f / sqrtf(ss / (float)Dv + eps);
     for (int j = threadIdx.x; j < Dv; j += WAVE) {
-        float g = gate ? to_f32(gate[row * Dv + j]) : 1.f;
-        if (gate_fn == 1) g = siluf_(g);
-        else if (gate_fn == 2) g = sigmoidf_(g);
-        y[row * Dv + j] = from_f32<T>(src[j] * inv * w[(long long)blockIdx.y * w_stride + j] * g);
+        const float wj = w[(long long)blockIdx.y * w_stride + j];
+        const float g = gate_of(j);
+        y[row * Dv + j] = from_f32<T>(gate_first ? (src[j] * g) * inv * wj : src[j] * inv * wj * g);
     }
 }
 
-template <typename TA, typename T, bool DELTA, bool FORGET = false>
+template <typename TA, typename T, bool DELTA, bool FORGET = false, bool SSD = false>
 int launch_scan(const ScanArgs& p, int R, hipStream_t stream) {
     if (p.H > 65535 || p.D > 256) return -2;
     const bool narrow = p.D <= 32;                      // four lanes a value channel; else sixteen
@@ -401,7 +446,7 @@ int launch_scan(const ScanArgs& p, int R, hipStream_t stream) {
     const int ni = narrow ? (p.D + 15) / 16 : (p.D + 63) / 64;
     dim3 grid(R, p.H, ceil_div(p.Dv, WAVE / split)), block(WAVE);
     if (grid.z > 65535) return -2;
-#define SCAN(NI, SPLIT) hipLaunchKernelGGL((scan_kernel<TA, T, NI, SPLIT, DELTA, FORGET>), grid, block, 0, stream, p)
+#define SCAN(NI, SPLIT) hipLaunchKernelGGL((scan_kernel<TA, T, NI, SPLIT, DELTA, FORGET, SSD>), grid, block, 0, stream, p)
     if (narrow) { if (ni <= 1) SCAN(1, 4); else SCAN(2, 4); }
     else if (ni <= 1) SCAN(1, 16);
     else if (ni <= 2) SCAN(2, 16);
@@ -432,20 +477,25 @@ TUFF_EXPORT int tuff_shift_state(const void* h, int dt, float* prev_state, const
     return launch_status();
 }
 
-// x, y [T][C]; taps float32 [C][K]; state float32 [slots][K-1][C].  q_len null: the state is only read.
-TUFF_EXPORT int tuff_conv_act(const void* x, int dt, const float* taps, float* state, void* y,
-                              const int* req_of_token, const int* q_start, const int* q_len, const int* state_slot,
+// x [T] rows of C channels ldx elements apart, of type dt; y [T][C] of type out_dt (where the types differ x is
+// float32); taps float32 [C][K]; bias float32 [C] or null; state float32 [slots][K-1][C].  q_len null: the state is
+// only read.
+TUFF_EXPORT int tuff_conv_act(const void* x, int dt, long long ldx, const float* taps, const float* bias, float* state, void* y,
+                              int out_dt, const int* req_of_token, const int* q_start, const int* q_len, const int* state_slot,
                               int n_tokens, int n_requests, int C, int K, int act, hipStream_t stream) {
     if (n_tokens <= 0) return 0;
-    if (K < 1 || K > MAX_TAPS) return -2;
+    if (K < 1 || K > MAX_TAPS || ldx < C || (dt != out_dt && dt != DT_F32)) return -2;
     const int cols = ceil_div(C, 256);
     dim3 block(256);
-    if (dt == DT_F32) hipLaunchKernelGGL(conv_act_kernel<float>, dim3(n_tokens, cols), block, 0, stream, (const float*)x, taps, state, (float*)y, req_of_token, q_start, state_slot, C, K, act);
-    else hipLaunchKernelGGL(conv_act_kernel<bf16_t>, dim3(n_tokens, cols), block, 0, stream, (const bf16_t*)x, taps, state, (bf16_t*)y, req_of_token, q_start, state_slot, C, K, act);
+#define CONV(T, TY) hipLaunchKernelGGL((conv_act_kernel<T, TY>), dim3(n_tokens, cols), block, 0, stream, (const T*)x, ldx, taps, bias, state, (TY*)y, req_of_token, q_start, state_slot, C, K, act)
+    if (dt == DT_F32 && out_dt == DT_F32) CONV(float, float);
+    else if (dt == DT_F32) CONV(float, bf16_t);
+    else CONV(bf16_t, bf16_t);
+#undef CONV
     int rc = launch_status();
     if (rc != 0 || !q_len || K == 1) return rc;
-    if (dt == DT_F32) hipLaunchKernelGGL(conv_state_kernel<float>, dim3(n_requests, cols), block, 0, stream, (const float*)x, state, q_start, q_len, state_slot, C, K);
-    else hipLaunchKernelGGL(conv_state_kernel<bf16_t>, dim3(n_requests, cols), block, 0, stream, (const bf16_t*)x, state, q_start, q_len, state_slot, C, K);
+    if (dt == DT_F32) hipLaunchKernelGGL(conv_state_kernel<float>, dim3(n_requests, cols), block, 0, stream, (const float*)x, ldx, state, q_start, q_len, state_slot, C, K);
+    else hipLaunchKernelGGL(conv_state_kernel<bf16_t>, dim3(n_requests, cols), block, 0, stream, (const bf16_t*)x, ldx, state, q_start, q_len, state_slot, C, K);
     return launch_status();
 }
 
@@ -456,7 +506,7 @@ TUFF_EXPORT int tuff_wkv_scan(const void* r, const void* k, const void* v, int d
                               const int* state_slot, int n_tokens, int n_requests, int H, int D, hipStream_t stream) {
     if (n_requests <= 0 || n_tokens <= 0) return 0;
     if (H > 65535) return -2;
-    PrepArgs pp{r, k, lw, w0, u, nullptr, nullptr, nullptr, bonus, H, H, D, (long long)H * D};
+    PrepArgs pp{r, k, lw, w0, u, nullptr, nullptr, 0, nullptr, nullptr, bonus, H, H, D, (long long)H * D};
     if (dt == DT_F32) hipLaunchKernelGGL((scan_prep_kernel<float, false>), dim3(n_tokens, H), dim3(WAVE), 0, stream, pp);
     else hipLaunchKernelGGL((scan_prep_kernel<bf16_t, false>), dim3(n_tokens, H), dim3(WAVE), 0, stream, pp);
     ScanArgs p{r, k, v, lw, bonus, state, out, q_start, q_len, state_slot, H, H, D, D, (long long)H * D};
@@ -466,15 +516,18 @@ TUFF_EXPORT int tuff_wkv_scan(const void* r, const void* k, const void* v, int d
 
 // delta: q, k (rows of Hk*D, ld elements apart) and v (rows of H*Dv, ldv apart) of type dt (they
 // may be parts of one wider row), after convolution and activation, not yet unit vectors; a float32
-// [T][H*D] (overwritten with the decays); dt_bias float32 [H*D]; A_log float32 [H]; b float32 [T][H]; work arrays
-// qn, kn float32 [T][H*D] and beta float32 [T][H]; state float32 [slots][H][D][Dv]; out float32 [T][H][Dv].
+// [T][H*D] (overwritten with the decays); dt_bias float32 [H*D]; A_log float32 [H]; b float32, a token's H values
+// ld_small apart; work arrays qn, kn float32 [T][H*D] and beta float32 [T][H]; state float32 [slots][H][D][Dv]; out
+// float32 [T][H][Dv].  a_head (or null): one decay per head, its inputs a token's H values ld_small apart, dt_bias
+// then [H]; a is then only written.
 TUFF_EXPORT int tuff_delta_scan(const void* q, const void* k, const void* v, int dt, float* a, const float* dt_bias,
-                                const float* A_log, const float* b, float* qn, float* kn, float* beta, float* state,
-                                float* out, const int* q_start, const int* q_len, const int* state_slot, int n_tokens,
-                                int n_requests, int H, int Hk, int D, int Dv, long long ld, long long ldv, hipStream_t stream) {
+                                const float* A_log, const float* b, const float* a_head, long long ld_small, float* qn, float* kn,
+                                float* beta, float* state, float* out, const int* q_start, const int* q_len, const int* state_slot,
+                                int n_tokens, int n_requests, int H, int Hk, int D, int Dv, long long ld, long long ldv,
+                                hipStream_t stream) {
     if (n_requests <= 0 || n_tokens <= 0) return 0;
-    if (Hk <= 0 || H % Hk || H > 65535) return -2;
-    PrepArgs pp{q, k, a, dt_bias, A_log, b, qn, kn, beta, H, Hk, D, ld};
+    if (Hk <= 0 || H % Hk || H > 65535 || ld_small < H) return -2;
+    PrepArgs pp{q, k, a, dt_bias, A_log, b, a_head, ld_small, qn, kn, beta, H, Hk, D, ld};
     if (dt == DT_F32) hipLaunchKernelGGL((scan_prep_kernel<float, true>), dim3(n_tokens, H), dim3(WAVE), 0, stream, pp);
     else hipLaunchKernelGGL((scan_prep_kernel<bf16_t, true>), dim3(n_tokens, H), dim3(WAVE), 0, stream, pp);
     ScanArgs p{qn, kn, v, a, beta, state, out, q_start, q_len, state_slot, H, H, D, Dv, ldv};
@@ -482,16 +535,39 @@ TUFF_EXPORT int tuff_delta_scan(const void* q, const void* k, const void* v, int
                         : launch_scan<float, bf16_t, true>(p, n_requests, stream);
 }
 
-// gate_dt: type of the gate's rows (float32 sums of a product may come in as they are); dt: type of y.
-TUFF_EXPORT int tuff_head_norm_gate(const float* o, const float* w, int w_stride, const void* gate, int gate_dt, int dt, int gate_fn,
-                                    void* y, int n_tokens, int H, int Dv, float eps, hipStream_t stream) {
+// gate_dt: type of the gate's rows (float32 sums of a product may come in as they are), gate_ld elements apart; dt:
+// type of y.  gate_first: the gate is applied before the norm.
+TUFF_EXPORT int tuff_head_norm_gate(const float* o, const float* w, int w_stride, const void* gate, long long gate_ld, int gate_dt,
+                                    int dt, int gate_fn, int gate_first, void* y, int n_tokens, int H, int Dv, float eps,
+                                    hipStream_t stream) {
     if (n_tokens <= 0) return 0;
+    if (H > 65535 || (gate && gate_ld < (long long)H * Dv)) return -2;
     dim3 grid(n_tokens, H), block(WAVE);
-    if (dt == DT_F32 && gate_dt == DT_F32) hipLaunchKernelGGL((head_norm_gate_kernel<float, float>), grid, block, 0, stream, o, w, w_stride, (const float*)gate, gate_fn, (float*)y, H, Dv, eps);
-    else if (gate_dt == DT_F32) hipLaunchKernelGGL((head_norm_gate_kernel<float, bf16_t>), grid, block, 0, stream, o, w, w_stride, (const float*)gate, gate_fn, (bf16_t*)y, H, Dv, eps);
-    else if (dt == DT_BF16) hipLaunchKernelGGL((head_norm_gate_kernel<bf16_t, bf16_t>), grid, block, 0, stream, o, w, w_stride, (const bf16_t*)gate, gate_fn, (bf16_t*)y, H, Dv, eps);
+    if (dt == DT_F32 && gate_dt == DT_F32) hipLaunchKernelGGL((head_norm_gate_kernel<float, float>), grid, block, 0, stream, o, w, w_stride, (const float*)gate, gate_ld, gate_fn, gate_first, (float*)y, H, Dv, eps);
+    else if (gate_dt == DT_F32) hipLaunchKernelGGL((head_norm_gate_kernel<float, bf16_t>), grid, block, 0, stream, o, w, w_stride, (const float*)gate, gate_ld, gate_fn, gate_first, (bf16_t*)y, H, Dv, eps);
+    else if (dt == DT_BF16) hipLaunchKernelGGL((head_norm_gate_kernel<bf16_t, bf16_t>), grid, block, 0, stream, o, w, w_stride, (const bf16_t*)gate, gate_ld, gate_fn, gate_first, (bf16_t*)y, H, Dv, eps);
     else return -2;
     return launch_status();
+}
+
+// ssd (the state-space recurrence with a scalar decay per head): xbc holds a token's convolved rows
+// [x (H*P) | B (G*N) | C (G*N)] of type dt, ld elements apart; dt_raw float32, a token's H values ld_dt apart; dt_bias,
+// A_log, Dh float32 [H]; work arrays qn, kn, decay float32 [T][H*N] and bonus float32 [T][H]; state float32
+// [slots][H][N][P]; out float32 [T][H][P].  Head h reads group h / (H / G).
+TUFF_EXPORT int tuff_ssd_scan(const void* xbc, int dt, long long ld, const float* dt_raw, long long ld_dt, const float* dt_bias,
+                              const float* A_log, const float* Dh, float* qn, float* kn, float* decay, float* bonus, float* state,
+                              float* out, const int* q_start, const int* q_len, const int* state_slot, int n_tokens, int n_requests,
+                              int H, int G, int N, int P, hipStream_t stream) {
+    if (n_requests <= 0 || n_tokens <= 0) return 0;
+    if (H <= 0 || H > 65535 || G <= 0 || H % G || ld < (long long)H * P + 2LL * G * N || ld_dt < H) return -2;
+    const int b_off = H * P;
+    if (dt == DT_F32) hipLaunchKernelGGL(ssd_prep_kernel<float>, dim3(n_tokens, H), dim3(WAVE), 0, stream, (const float*)xbc, ld, b_off, dt_raw, ld_dt, dt_bias, A_log, Dh, qn, kn, decay, bonus, H, G, N);
+    else hipLaunchKernelGGL(ssd_prep_kernel<bf16_t>, dim3(n_tokens, H), dim3(WAVE), 0, stream, (const bf16_t*)xbc, ld, b_off, dt_raw, ld_dt, dt_bias, A_log, Dh, qn, kn, decay, bonus, H, G, N);
+    int rc = launch_status();
+    if (rc != 0) return rc;
+    ScanArgs p{qn, kn, xbc, decay, bonus, state, out, q_start, q_len, state_slot, H, H, N, P, ld};
+    return dt == DT_F32 ? launch_scan<float, float, false, false, true>(p, n_requests, stream)
+                        : launch_scan<float, bf16_t, false, false, true>(p, n_requests, stream);
 }
 
 // forget: x rows [q (H*D) | z (H*D) | v (H*Dv)] of type dt, ld elements apart, as projected; bias (or null) and lower

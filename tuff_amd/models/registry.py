@@ -77,6 +77,9 @@ def _register_builtin() -> None:
     from ..config.loluzen import LoluzenConfig
     from .loluzen import build_loluzen
     register_architecture(LoluzenConfig.architecture, LoluzenConfig, build_loluzen)
+    from ..config.kinelix import KinelixConfig
+    from .kinelix import build_kinelix
+    register_architecture(KinelixConfig.architecture, KinelixConfig, build_kinelix)
 
 
 _register_builtin()

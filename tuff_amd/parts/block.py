@@ -10,6 +10,9 @@ ParallelBlock has one norm whose output both sublayers read:
 SandwichBlock norms a sublayer on both sides:
     x += m * norm1b(mixer(norm1(x)));  x += m * norm2b(ffn(norm2(x)))
 
+LayerScaleBlock is the pre-norm layer whose sublayers' outputs are scaled per channel before they join the stream:
+    x += ls1 * mixer(norm1(x));  x += ls2 * ffn(norm2(x))
+
 HyperConnectionBlock is the pre-norm layer over several residual streams: a sublayer reads a weighted sum
 of the streams and its output goes back into all of them through a mixing matrix.
 """
@@ -21,7 +24,7 @@ import torch
 
 from ..csrc import ops
 from .base import BLOCKS, Block, FeedForward, Mixer, Norm, Runtime, WeightDecl
-from .norm import RMSNorm
+from .norm import LayerNorm, RMSNorm
 
 
 @BLOCKS.register("prenorm")
@@ -221,6 +224,93 @@ class SandwichBlock(Block):
             h = self.rt.empty(*x.shape)
             kw = dict(next_w=read[0], next_eps=read[1], h_out=h)
         ops.post_norm_add(x, y=y, w=after.weight_f32, eps=after.eps, mult=self.mult, extra=extra, clear_y=True, y_next=y_next, **kw)
+        return h
+
+
+@BLOCKS.register("layer_scale")
+class LayerScaleBlock(Block):
+    """x <- x + ls1 * mixer(norm1(x)), then x <- x + ls2 * ffn(norm2(x)): pre-norm with a learned scale per channel
+    ('layer scale') on each sublayer's output.  ffn None: the mixer's sublayer alone.  The norms are layer norms (they
+    run inside one kernel, ops.scale_add_layer_norm, which scales a sublayer's output, adds it into the stream and
+    reads the next sublayer's input with its norm; the next sublayer may be the next block's first, so forward()
+    takes what the block before left (`carry`) and is told who reads next (`next_read`)).  names: checkpoint names
+    'ls1' [d] and, with a feed-forward, 'ls2' [d]."""
+    carries_norm = True
+
+    def __init__(self, norm1: Norm, mixer: Mixer, norm2: Optional[Norm] = None, ffn: Optional[FeedForward] = None, *,
+                 names: dict[str, str]):
+        if (norm2 is None) != (ffn is None):
+            raise ValueError("norm2 and ffn go together")
+        for n in (norm1, norm2):
+            if n is not None and not isinstance(n, LayerNorm):
+                raise ValueError("the norms of a layer-scale block are layer norms (they run inside the block's kernel)")
+        self.norm1, self.mixer, self.norm2, self.ffn = norm1, mixer, norm2, ffn
+        self.names = dict(names)
+
+    def _parts(self):
+        return [p for p in (self.norm1, self.mixer, self.norm2, self.ffn) if p is not None]
+
+    @property
+    def graph_safe(self):
+        return all(p.graph_safe for p in self._parts())
+
+    @property
+    def records_portions(self):
+        return all(p.records_portions for p in self._parts())
+
+    def weight_decls(self):
+        decls = [d for p in self._parts() for d in p.weight_decls()]
+        decls.append(WeightDecl(self.names["ls1"], (self.norm1.dim,), "norm"))
+        if self.ffn is not None:
+            decls.append(WeightDecl(self.names["ls2"], (self.norm1.dim,), "norm"))
+        return decls
+
+    def kernel_modules(self):
+        return ["postnorm", "elementwise"] + [m for p in self._parts() for m in p.kernel_modules()]
+
+    def token_inputs(self):
+        return [t for p in self._parts() for t in p.token_inputs()]
+
+    def bind(self, weights, rt: Runtime):
+        self.rt = rt
+        for p in self._parts():
+            p.bind(weights, rt)
+        self.ls1 = weights[self.names["ls1"]].float().contiguous()
+        self.ls2 = weights[self.names["ls2"]].float().contiguous() if self.ffn is not None else None
+
+    def first_read(self):
+        """(norm weight float32 [d], eps): what the block before needs to prepare this block's first input."""
+        return self.norm1.weight_f32, self.norm1.eps
+
+    def forward(self, x, ctx, cache, write_cache: bool = True, carry=None, next_read=None, y=None, extra=None):
+        """x float32 [T, d], in place.  carry: norm1(x) where the block before left it (None: computed here).
+        next_read: (norm weight, eps) of whoever reads x next; that norm of the new x is returned (None: nothing is
+        read and None returned).  y: float32 [T, d] of zeros that the sublayers add into (left zero again); None:
+        made here."""
+        if extra is not None:
+            raise ValueError("a layer-scale block adds nothing but its sublayers to the stream")
+        T, d = x.shape
+        if carry is None:
+            carry = self.norm1.forward(x)
+        if y is None:
+            y = torch.empty(T, d, dtype=torch.float32, device=x.device)
+            ops.fill_u32(y, 0)
+        kw = {"next_norm": None} if self.mixer.adds_once_through_linear else {}
+        self.mixer.forward(carry, ctx, cache, y, write_cache, **kw)
+        if self.ffn is None:
+            return self._join(x, y, self.ls1, next_read)
+        h = self._join(x, y, self.ls1, (self.norm2.weight_f32, self.norm2.eps))
+        kw = {"next_norm": None} if self.ffn.adds_once_through_linear else {}
+        self.ffn.forward(h, ctx, y, **kw)
+        return self._join(x, y, self.ls2, next_read)
+
+    def _join(self, x, y, ls, read):
+        h = None
+        kw = {}
+        if read is not None:
+            h = self.rt.empty(*x.shape)
+            kw = dict(next_w=read[0], eps=read[1], h_out=h)
+        ops.scale_add_layer_norm(x, y=y, ls=ls, clear_y=True, **kw)
         return h
 
 

@@ -215,17 +215,33 @@ class MoE(FeedForward):
     gated: an expert is W_down glu(W_gate x, W_up x) and 'experts' lists (gate, up, down) names; glu(g, u) is
     act(g) u, or, activation "swish_clamp", g' sigmoid(alpha g') (u' + 1) with g' = min(g, limit) and
     u' = clamp(u, -limit, limit).  shared: a feed-forward of any kind that runs for every token and is added (in
-    place of the built-in ungated one that shared_dim asks for)."""
+    place of the built-in ungated one that shared_dim asks for).
+    A limited choice (router_weights "sigmoid"; switched on by route_groups, a name 'correction' or route_scale): the
+    choice runs on sigmoid(z) + correction ('correction' [E], which the weights do not see) and only inside the
+    route_keep groups, of route_groups equal groups of neighbouring experts, whose two largest such scores have the
+    largest sum (an expert outside them cannot be chosen, whatever its score); the weights are the chosen experts'
+    sigmoid(z) times route_scale, not renormalised."""
     graph_safe = True
     records_portions = True
 
     def __init__(self, hidden_size: int, num_experts: int, top: int, expert_dim: int, *, names: dict,
                  activation: str = "relu2", router_weights: str = "sigmoid", scale_input: bool = True,
                  shared_dim: int = 0, gated: bool = False, limit: float = 0.0, alpha: float = 1.0,
-                 shared: FeedForward | None = None):
+                 shared: FeedForward | None = None, route_groups: int = 0, route_keep: int = 0, route_scale: float = 1.0):
         self.d, self.E, self.top, self.F = int(hidden_size), int(num_experts), int(top), int(expert_dim)
         if not 1 <= self.top <= self.E:
             raise ValueError(f"top {self.top} of {self.E} experts")
+        self.has_correction = "correction" in names
+        self.route_scale = float(route_scale)
+        self.route_groups, self.route_keep = int(route_groups), int(route_keep)
+        if not self.route_groups and (self.has_correction or self.route_scale != 1.0):
+            self.route_groups = self.route_keep = 1              # one group of all experts, kept: the choice is not limited
+        if self.route_groups:
+            G, keep = self.route_groups, self.route_keep
+            if router_weights != "sigmoid" or "router.b" in names:
+                raise ValueError("a limited choice goes with sigmoid weights and no bias on the logits")
+            if not 1 <= G <= 64 or self.E % G or not 1 <= keep <= G or self.top > keep * (self.E // G):
+                raise ValueError(f"top {self.top} among {keep} of {G} groups of {self.E} experts")
         if activation not in ("relu2", "silu", "gelu_tanh", "swish_clamp"):
             raise ValueError(f"unknown activation '{activation}'")
         self.gated, self.limit, self.alpha = bool(gated), float(limit), float(alpha)
@@ -255,6 +271,8 @@ class MoE(FeedForward):
             decls.append(WeightDecl(self.names["shared.sg"], (1, self.d), "normal", role="projection"))
         if self.has_router_bias:
             decls.append(WeightDecl(self.names["router.b"], (self.E,), "normal"))
+        if self.has_correction:
+            decls.append(WeightDecl(self.names["correction"], (self.E,), "normal"))
         for e in self.names["experts"]:
             decls += [WeightDecl(n, (self.F, self.d), "normal", role="projection") for n in e[:-1]]
             decls.append(WeightDecl(e[-1], (self.d, self.F), "normal", role="projection"))
@@ -274,6 +292,7 @@ class MoE(FeedForward):
         rows = [weights[self.names["router"]]] + ([weights[self.names["shared.sg"]]] if self.shared_gate else [])
         self.router_w = torch.cat([r.to(torch.float32).reshape(-1, self.d) for r in rows]).contiguous()
         self.router_b = weights[self.names["router.b"]].to(torch.float32).contiguous() if self.has_router_bias else None
+        self.correction = weights[self.names["correction"]].to(torch.float32).contiguous() if self.has_correction else None
         ups = [weights[e[-2]] for e in self.names["experts"]]
         gates = [weights[e[0]] for e in self.names["experts"]] if self.gated else None
         downs = [weights[e[-1]] for e in self.names["experts"]]
@@ -306,7 +325,8 @@ class MoE(FeedForward):
         z = torch.empty(T, self.router_w.shape[0], dtype=torch.float32, device=h.device)        # [T, E (+ 1)]
         ids = torch.empty(T, self.top, dtype=torch.int32, device=h.device)
         wts = torch.empty(T, self.top, dtype=torch.float32, device=h.device)
-        ops.moe_router(h, self.router_w, z, ids, wts, E=self.E, top=self.top, weights=self.router_weights, bias=self.router_b)
+        ops.moe_router(h, self.router_w, z, ids, wts, E=self.E, top=self.top, weights=self.router_weights, bias=self.router_b,
+                       correction=self.correction, groups=self.route_groups, keep=self.route_keep, scale=self.route_scale)
         form = dict(activation=self.activation, scale_input=self.scale_input, gated=self.gated, limit=self.limit, alpha=self.alpha)
         if self.grouped:
             ops.moe_experts_grouped(h, self.up_tiles, self.down_tiles, ids, wts, residual, F=self.F, **form)

@@ -3,6 +3,7 @@
 RMSNorm: y = x / sqrt(mean(x^2) + eps) * w (src/lfm25_gpu.cu:235,244); with offset c the stored weight
 lies around zero and y = x / sqrt(mean(x^2) + eps) * (c + w).
 DynamicTanh: y = tanh(alpha x) w + b with a learned scalar alpha; no mean, no variance.
+LayerNorm: y = (x - mean) / sqrt(mean((x - mean)^2) + eps) * w, a weight and no bias.
 """
 from __future__ import annotations
 
@@ -118,4 +119,31 @@ class DynamicTanh(Norm):
         n = x.shape[0] if rows is None else rows.shape[0]
         out = self.rt.empty(n, self.dim)
         ops.dyt(x, self.weight_f32, self.bias_f32, self.alpha_f32, out, rows)
+        return out
+
+
+@NORMS.register("layernorm")
+class LayerNorm(Norm):
+    """y = (x - mean(x)) / sqrt(var(x) + eps) * w with var the mean of the squared deviations; a weight [d] and no
+    bias.  Statistics and result are formed in float32 and rounded once to the compute type."""
+    graph_safe = True
+    records_portions = True
+
+    def __init__(self, dim: int, eps: float, name: str):
+        self.dim, self.eps, self.name = int(dim), float(eps), name
+
+    def weight_decls(self):
+        return [WeightDecl(self.name, (self.dim,), "norm")]
+
+    def kernel_modules(self):
+        return ["postnorm"]
+
+    def bind(self, weights, rt: Runtime):
+        self.rt = rt
+        self.weight_f32 = weights[self.name].float().contiguous()
+
+    def forward(self, x: torch.Tensor, rows: Optional[torch.Tensor] = None) -> torch.Tensor:
+        n = x.shape[0] if rows is None else rows.shape[0]
+        out = self.rt.empty(n, self.dim)
+        ops.scale_add_layer_norm(x, next_w=self.weight_f32, eps=self.eps, h_out=out, rows=rows)
         return out
