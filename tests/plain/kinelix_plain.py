@@ -143,10 +143,14 @@ def dense_ff(n, W, rnd=_same):
     return rnd(silu(n @ W["gate"].T) * (n @ W["up"].T)) @ W["down"].T
 
 
-def route(n, W, spec):
+def route(n, W, spec, margins_out=None):
     """ids [T, top] and weights [T, top].  Scores are sigmoid(W_router n); the choice runs on score + correction,
     only inside the groups.keep groups whose two largest choice scores have the largest sum; the weights are the
-    chosen experts' plain scores times router.scale, not renormalised.  Ties go to the lower index."""
+    chosen experts' plain scores times router.scale, not renormalised.  Ties go to the lower index.
+    margins_out: a list that receives, per token, the smaller of two gaps, each as a share of the root mean square of
+    all the sequence's choice scores about their mean: between the last kept group's score and the first dropped one's,
+    and between the last chosen expert's choice score and the first one left out inside the kept groups (infinite
+    where nothing is left out)."""
     r = spec["router"]
     E, top = r["experts"], r["top"]
     count, keep = r["groups"]["count"], r["groups"]["keep"]
@@ -155,6 +159,8 @@ def route(n, W, spec):
     T = n.shape[0]
     per = E // count
     ids = torch.zeros(T, top, dtype=torch.long)
+    margins = torch.full((T,), math.inf, dtype=F64)
+    spread = (choice - choice.mean()).pow(2).mean().sqrt().clamp_min(1e-30)
     for t in range(T):
         grp = []
         for g in range(count):
@@ -164,13 +170,20 @@ def route(n, W, spec):
         allowed = [e for e in range(E) if e // per in kept]
         order = sorted(allowed, key=lambda e: (-choice[t, e].item(), e))
         ids[t] = torch.tensor(order[:top])
+        by_score = sorted(grp, reverse=True)
+        if keep < count:
+            margins[t] = min(margins[t], (by_score[keep - 1] - by_score[keep]) / spread)
+        if top < len(order):
+            margins[t] = min(margins[t], (choice[t, order[top - 1]] - choice[t, order[top]]) / spread)
+    if margins_out is not None:
+        margins_out.append(margins)
     wts = torch.gather(s, 1, ids) * r["scale"]
     return ids, wts
 
 
-def moe_ff(n, W, spec, rnd=_same):
+def moe_ff(n, W, spec, rnd=_same, margins_out=None):
     T, d = n.shape
-    ids, wts = route(n, W, spec)
+    ids, wts = route(n, W, spec, margins_out)
     out = torch.zeros(T, d, dtype=F64)
     for t in range(T):
         for e, w in zip(ids[t].tolist(), wts[t]):
@@ -184,8 +197,9 @@ def _sub(weights, prefix):
     return {k[len(prefix):]: v.to(F64) for k, v in weights.items() if k.startswith(prefix)}
 
 
-def forward(cfg: dict, weights: dict, tokens, rnd=_same, on_layer=None) -> torch.Tensor:
-    """Logits [T, vocab] of one sequence.  on_layer(i, x): called with the residual stream after every layer."""
+def forward(cfg: dict, weights: dict, tokens, rnd=_same, on_layer=None, margins_out=None) -> torch.Tensor:
+    """Logits [T, vocab] of one sequence.  on_layer(i, x): called with the residual stream after every layer.
+    margins_out: see route()."""
     eps = cfg["norm"]["eps"]
     tokens = torch.as_tensor(tokens, dtype=torch.long)
     x = weights["embed"].to(F64)[tokens] * cfg["embedding"]["scale"]
@@ -209,7 +223,7 @@ def forward(cfg: dict, weights: dict, tokens, rnd=_same, on_layer=None) -> torch
         if spec is not None:
             n = rnd(layer_norm(x, weights[f"l{i}.norm2"].to(F64), eps))
             Wf = _sub(weights, f"l{i}.mlp.")
-            y = dense_ff(n, Wf, rnd) if spec["kind"] == "dense" else moe_ff(n, Wf, spec, rnd)
+            y = dense_ff(n, Wf, rnd) if spec["kind"] == "dense" else moe_ff(n, Wf, spec, rnd, margins_out)
             x = x + y * weights[f"l{i}.ls2"].to(F64)
         if on_layer is not None:
             on_layer(i, x)
