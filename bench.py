@@ -393,6 +393,30 @@ def loluzen_config(size: str):
                              "norm": {"eps": 1e-5}, "residual_mult": 0.5, "layers": [kinds[i % 2] for i in range(L)]})
 
 
+def kinelix_config(size: str):
+    """`--design kinelix`: the layer order repeats [mamba2 + dense, latent attention + experts, delta + dense, latent
+    attention on the rows of the layer two before + experts]; mamba2 with twice the width inside in heads of 64, a state
+    of 128 and 8 groups, the delta rule with keys of 64 and values of 128 a head, latent attention with heads of 64 on a
+    row of 192, experts chosen inside 2 of 4 groups."""
+    from tuff_amd.models.registry import config_from_dict
+    d, L, H, G, ff, E, top, eff = DESIGN_SIZES[size]
+    dense = {"kind": "dense", "ff": ff}
+    moe = {"kind": "moe", "router": {"experts": E, "top": top, "scale": 1.5, "groups": {"count": 4, "keep": 2}}, "expert": {"ff": eff}}
+    latent = {"heads": H, "dim": 64, "vdim": 64, "kv_rank": 192, "scale": 0.125}
+    layers = []
+    for i in range(L):
+        kind = i % 4
+        if kind == 0:
+            layers.append({"type": "mamba2", "mixer": {"heads": 2 * d // 64, "vdim": 64, "state": 128, "groups": 8, "norm_groups": 8,
+                                                       "conv": 4}, "mlp": dense})
+        elif kind == 2:
+            layers.append({"type": "delta", "mixer": {"heads": H // 2, "kv_heads": H // 4, "dim": 64, "vdim": 128, "conv": 4}, "mlp": dense})
+        else:
+            layers.append({"type": "latent_attention", "mixer": dict(latent, **({"kv_from": i - 2} if kind == 3 else {})), "mlp": moe})
+    return config_from_dict({"architecture": "Kinelix", "vocab": DESIGN_VOCAB, "width": d, "embedding": {"scale": 1.0},
+                             "norm": {"eps": 1e-5}, "logit_softcap": 30.0, "layers": layers})
+
+
 def lfm2_config_like(size: str, attention_every: int = 4):
     """The LFM2 model of the same width, depth, heads, vocabulary and dense feed-forward: its short-conv
     layers stand where the other design has its recurrences (attention_every 1: attention in every layer, beside a
@@ -473,11 +497,12 @@ def time_design(cfg, dtype: str, prefill_tokens: int, batch: int, context: int, 
 
 
 def run_design(args) -> dict:
-    """`--design pafodra|kugalorn|loluzen`: that decoder at sizes that resemble a real model's layers (random weights)
+    """`--design pafodra|kugalorn|loluzen|kinelix`: that decoder at sizes that resemble a real model's layers (random weights)
     beside the LFM2 decoder of equal width, depth and feed-forward."""
     dtype = "bfloat16" if args.dtype == "bf16" else "float32"
     classes = os.environ.get("TUFF_TRACE", "")[:1] == "1"
-    design, make = args.design, {"pafodra": pafodra_config, "kugalorn": kugalorn_config, "loluzen": loluzen_config}[args.design]
+    design, make = args.design, {"pafodra": pafodra_config, "kugalorn": kugalorn_config, "loluzen": loluzen_config,
+                                 "kinelix": kinelix_config}[args.design]
     every = 1 if design == "loluzen" else 4
     out = {"design": design, "dtype": args.dtype, "prefill_tokens": PREFILL_TOKENS, "decode_batch": args.batch,
            "decode_context": args.design_context, "data": f"synthetic: seeded random weights (seed {SEED}), uniform random token ids",
@@ -570,7 +595,7 @@ def main() -> int:
     ap.add_argument("--shape", default="1.2b", choices=["1.2b"] + sorted(OTHER_SHAPES),
                     help="measure another shape of the architecture in the benchmark's place (for profiling; "
                          "its points only, no other shapes after it)")
-    ap.add_argument("--design", choices=["pafodra", "kugalorn", "loluzen"],
+    ap.add_argument("--design", choices=["pafodra", "kugalorn", "loluzen", "kinelix"],
                     help="instead of the benchmark: prefill and decode of another design at sizes that resemble a real "
                          "model's layers, beside the LFM2 model of equal size (TUFF_TRACE=1 adds GPU time by kernel class)")
     ap.add_argument("--design-sizes", default="1k,2k", help="with --design: which of " + ",".join(sorted(DESIGN_SIZES)))

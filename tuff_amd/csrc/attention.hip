@@ -226,10 +226,11 @@ __global__ __launch_bounds__(DEC_KEYS) void decode_scores_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_cache, float* __restrict__ S, float* __restrict__ ml,
     const int* __restrict__ block_table, int max_blocks, const int* __restrict__ req_of_token, const int* __restrict__ positions,
     int H, int Hkv, int hd, int page_size, int window, float scale, const float* __restrict__ slopes,
-    const float* __restrict__ log_r1, const float* __restrict__ log_r2, int n_parts) {
+    const float* __restrict__ log_r1, const float* __restrict__ log_r2, int n_parts, int chunks) {
     __shared__ float qs[DEC_HEADS * 256];
     __shared__ float scratch[4];
-    const int t = blockIdx.x, kvh = blockIdx.y, part = blockIdx.z, tid = threadIdx.x;
+    // (a group of more than GC heads is shared out among `chunks` workgroups, GC heads at a time each)
+    const int t = blockIdx.x, kvh = blockIdx.y / chunks, chunk = blockIdx.y % chunks, part = blockIdx.z, tid = threadIdx.x;
     const int G = H / Hkv;
     const int pos = positions[blockIdx.x];
     const int lo = (window > 0) ? max(0, pos - window + 1) : 0;
@@ -242,7 +243,7 @@ __global__ __launch_bounds__(DEC_KEYS) void decode_scores_kernel(
         krow = k_cache + ((page * Hkv + kvh) * page_size + key % page_size) * hd;
     }
     const float dist = (float)(pos - key);
-    for (int g0 = 0; g0 < G; g0 += GC) {
+    for (int g0 = chunk * GC; g0 < G; g0 += chunks * GC) {
         const int Gc = min(GC, G - g0);
         const int head0 = kvh * G + g0;
         if (!part_live) {                                       // uniform: no key of the part is visible
@@ -309,10 +310,12 @@ template <int GC>
 __global__ __launch_bounds__(DEC_KEYS) void decode_values_kernel(
     const float* __restrict__ S, const float* __restrict__ ml, const bf16_t* __restrict__ v_cache, float* __restrict__ po,
     const int* __restrict__ block_table, int max_blocks, const int* __restrict__ req_of_token, const int* __restrict__ positions,
-    int H, int Hkv, int vd, int page_size, int window, const float* __restrict__ sinks, const float* __restrict__ talk, int n_parts) {
+    int H, int Hkv, int vd, int page_size, int window, const float* __restrict__ sinks, const float* __restrict__ talk, int n_parts,
+    int chunks) {
     __shared__ float m_all[DEC_MAX_H], inv_all[DEC_MAX_H];
     __shared__ float w[DEC_HEADS * DEC_KEYS];                 // weights [head of the group][key]; then the slices' sums
-    const int t = blockIdx.x, kvh = blockIdx.y, part = blockIdx.z, tid = threadIdx.x;
+    const int t = blockIdx.x, kvh = blockIdx.y / chunks, chunk = blockIdx.y % chunks, part = blockIdx.z, tid = threadIdx.x;
+    const int g_first = chunk * GC;                           // the first heads of the group this workgroup takes
     const int G = H / Hkv;
     const int pos = positions[blockIdx.x];
     const int lo = (window > 0) ? max(0, pos - window + 1) : 0;
@@ -330,7 +333,7 @@ __global__ __launch_bounds__(DEC_KEYS) void decode_values_kernel(
     float s_first[GC];
 #pragma unroll
     for (int g = 0; g < GC; ++g)
-        s_first[g] = (!talk && valid && g < G) ? S[((long long)t * H + kvh * G + g) * n_parts * DEC_KEYS + key] : -INFINITY;
+        s_first[g] = (!talk && valid && g_first + g < G) ? S[((long long)t * H + kvh * G + g_first + g) * n_parts * DEC_KEYS + key] : -INFINITY;
     // every head's maximum and sum over the parts (all heads with a mixing matrix, else the group's)
     const int h_first = talk ? 0 : kvh * G, h_count = talk ? H : G;
     // (eight lanes a head, each a share of the parts, so that the loads are in flight together)
@@ -366,7 +369,7 @@ __global__ __launch_bounds__(DEC_KEYS) void decode_values_kernel(
     const int slices = max(1, DEC_KEYS / vd);                   // threads (channel, slice of the part's pages)
     const int d = tid % vd, sl = tid / vd;
     const bool works = tid < vd * slices;
-    for (int g0 = 0; g0 < G; g0 += GC) {
+    for (int g0 = g_first; g0 < G; g0 += chunks * GC) {
         const int Gc = min(GC, G - g0);
         const int head0 = kvh * G + g0;
         __syncthreads();
@@ -394,7 +397,7 @@ __global__ __launch_bounds__(DEC_KEYS) void decode_values_kernel(
 #pragma unroll
                 for (int g = 0; g < GC; ++g)
                     if (g < Gc) {
-                        const float sc = g0 == 0 ? s_first[g] : S[((long long)t * H + head0 + g) * n_parts * DEC_KEYS + key];
+                        const float sc = g0 == g_first ? s_first[g] : S[((long long)t * H + head0 + g) * n_parts * DEC_KEYS + key];
                         wk[g] = expf(sc - m_all[g0 + g]) * inv_all[g0 + g];
                     }
             }
@@ -496,13 +499,18 @@ TUFF_EXPORT int tuff_attention_decode_exact(const void* q, const void* k_cache, 
     if (Hkv <= 0 || H % Hkv != 0 || H > DEC_MAX_H || hd % 8 != 0 || hd > 256 || vd <= 0 || vd > DEC_KEYS) return -2;
     if (page_size % 8 != 0 || DEC_KEYS % page_size != 0 || n_parts <= 0 || n_parts > 65535 || Hkv > 65535) return -2;
     if ((log_r1 == nullptr) != (log_r2 == nullptr) || !S || !ml || !po) return -2;
-    dim3 grid(n_tokens, Hkv, n_parts), block(DEC_KEYS);
+    // a group of more than sixteen heads (one row a position for every head, as latent attention has) is shared out
+    // among several workgroups, sixteen heads each: the keys and values come from the caches once more, the step's few
+    // workgroups become as many more
+    const int chunks = (H / Hkv + DEC_HEADS - 1) / DEC_HEADS;
+    if ((long long)Hkv * chunks > 65535) return -2;
+    dim3 grid(n_tokens, Hkv * chunks, n_parts), block(DEC_KEYS);
     // (the loops over a group's heads are unrolled to the power of two that holds them, sixteen at most)
 #define LAUNCH(GC) do { \
     hipLaunchKernelGGL(decode_scores_kernel<GC>, grid, block, 0, stream, (const bf16_t*)q, (const bf16_t*)k_cache, S, ml, block_table, \
-                       max_blocks, req_of_token, positions, H, Hkv, hd, page_size, window, scale, slopes, log_r1, log_r2, n_parts); \
+                       max_blocks, req_of_token, positions, H, Hkv, hd, page_size, window, scale, slopes, log_r1, log_r2, n_parts, chunks); \
     hipLaunchKernelGGL(decode_values_kernel<GC>, grid, block, 0, stream, (const float*)S, (const float*)ml, (const bf16_t*)v_cache, po, \
-                       block_table, max_blocks, req_of_token, positions, H, Hkv, vd, page_size, window, sinks, talk, n_parts); } while (0)
+                       block_table, max_blocks, req_of_token, positions, H, Hkv, vd, page_size, window, sinks, talk, n_parts, chunks); } while (0)
     const int G = H / Hkv;
     if (G <= 1) LAUNCH(1); else if (G <= 2) LAUNCH(2); else if (G <= 4) LAUNCH(4); else if (G <= 8) LAUNCH(8); else LAUNCH(16);
 #undef LAUNCH

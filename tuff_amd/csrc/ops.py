@@ -54,8 +54,8 @@ _SIGNATURES = {
                             _c_int, _c_int, _c_int, _c_ll, _c_ll, _c_void_p],
         "tuff_head_norm_gate": [_c_void_p, _c_void_p, _c_int, _c_void_p, _c_ll, _c_int, _c_int, _c_int, _c_int, _c_void_p, _c_int, _c_int,
                                 _c_int, _c_float, _c_void_p],
-        "tuff_ssd_scan": [_c_void_p, _c_int, _c_ll, _c_void_p, _c_ll, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p,
-                          _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int,
+        "tuff_ssd_scan": [_c_void_p, _c_int, _c_ll, _c_void_p, _c_ll, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p,
+                          _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int,
                           _c_int, _c_void_p],
         "tuff_forget_scan": [_c_void_p, _c_int, _c_ll, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p,
                              _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p],
@@ -1635,11 +1635,11 @@ def ssd_scan(xbc, dt_raw, dt_bias, A_log, D_skip, state, out, *, q_start, q_len,
     ld_dt = _rows_view("dt_raw", dt_raw, H)
     if dt_raw.dtype != torch.float32:
         raise KernelError("ssd_scan: dt_raw must be float32")
-    work = torch.empty(3, T, H * N, dtype=torch.float32, device=xbc.device)     # queries, keys, decays
+    work = torch.empty(2, T, H, dtype=torch.float32, device=xbc.device)     # step sizes and decays
     _check(load("recurrent").tuff_ssd_scan(
         xbc.data_ptr(), _dt(xbc), ld, dt_raw.data_ptr(), ld_dt, _gpu("dt_bias", dt_bias, torch.float32, (H,)),
         _gpu("A_log", A_log, torch.float32, (H,)), _gpu("D_skip", D_skip, torch.float32, (H,)),
-        work[0].data_ptr(), work[1].data_ptr(), work[2].data_ptr(), torch.empty(T, H, dtype=torch.float32, device=xbc.device).data_ptr(),
+        work[0].data_ptr(), work[1].data_ptr(),
         _gpu("state", state, torch.float32, (None, H, N, P)), _gpu("out", out, torch.float32, (T, H * P)),
         _gpu("q_start", q_start, torch.int32, (R,)), _gpu("q_len", q_len, torch.int32, (R,)),
         _gpu("state_slot", state_slot, torch.int32, (R,)), T, R, H, G, N, P, _stream()), "ssd_scan")

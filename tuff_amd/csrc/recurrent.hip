@@ -192,41 +192,31 @@ __global__ void forget_prep_kernel(const T* __restrict__ x, long long ld, const 
     }
 }
 
-// What enters the state-space recurrence of head h (group g = h / (H / G)) at token t, all float32:
-// dt = softplus(dt_raw + dt_bias_h), decay = exp(-exp(A_log_h) dt) (the same for all N state channels),
-// key = dt B[t][g], query = C[t][g], and the head's D as the bonus on the token's own input.
-// bc: a token's convolved rows [.. | B (G*N) | C (G*N)] of type T, ldbc apart, B from column b_off.
+// What enters the state-space recurrence besides the convolved rows, float32 [T][H] each: the step size
+// dt = softplus(dt_raw + dt_bias_h) and the decay exp(-exp(A_log_h) dt), one number for all state channels of a head.
 // dt_raw float32, a token's H values ld_dt apart.
-template <typename T>
-__global__ __launch_bounds__(WAVE) void ssd_prep_kernel(const T* __restrict__ bc, long long ldbc, int b_off, const float* __restrict__ dt_raw,
-                                                        long long ld_dt, const float* __restrict__ dt_bias, const float* __restrict__ A_log,
-                                                        const float* __restrict__ Dh, float* __restrict__ qn, float* __restrict__ kn,
-                                                        float* __restrict__ decay, float* __restrict__ scalar, int H, int G, int N) {
-    const long long t = blockIdx.x;
-    const int head = blockIdx.y, lane = threadIdx.x;
-    const int g = head / (H / G);
+__global__ void ssd_prep_kernel(const float* __restrict__ dt_raw, long long ld_dt, const float* __restrict__ dt_bias,
+                                const float* __restrict__ A_log, float* __restrict__ dt_out, float* __restrict__ decay, long long n, int H) {
+    const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    const long long t = i / H;
+    const int head = (int)(i % H);
     const float dt = softplusf_(dt_raw[t * ld_dt + head] + dt_bias[head]);
-    const float dec = expf(-expf(A_log[head]) * dt);
-    const T* pb = bc + t * ldbc + b_off + (long long)g * N;
-    const T* pc = pb + (long long)G * N;
-    const long long o = (t * H + head) * N;
-    for (int i = lane; i < N; i += WAVE) {
-        kn[o + i] = dt * to_f32(pb[i]);
-        qn[o + i] = to_f32(pc[i]);
-        decay[o + i] = dec;
-    }
-    if (lane == 0) scalar[t * H + head] = Dh[head];
+    dt_out[i] = dt;
+    decay[i] = expf(-expf(A_log[head]) * dt);
 }
 
 struct ScanArgs {
-    const void *a, *k, *v;          // per token: a (r, or unit q) and k [T][Ha*D]; v: rows of H*Dv, ldv apart   (Ha: heads of a and k)
-    const float* decay;             // per token [T][H*D]: w or g
-    const float* scalar;            // per token [T][H]: bonus or beta
+    const void *a, *k, *v;          // per token: a (r, or unit q) and k, rows of Ha*D, lda apart; v: rows of H*Dv, ldv apart   (Ha: heads of a and k)
+    const float* decay;             // per token [T][H*D]: w or g; ssd: [T][H], one decay for all of a head's key channels
+    const float* scalar;            // per token [T][H]: bonus or beta; ssd: the step size dt, which multiplies the key
     float* state;                   // [slots][H][D][Dv]
     float* out;                     // [T][H][Dv]
     const int *q_start, *q_len, *state_slot;
     int H, Ha, D, Dv;
     long long ldv;                  // elements between two tokens' rows of v
+    long long lda;                  // elements between two tokens' rows of a and k
+    const float* head_bonus;        // ssd: [H], the factor of the token's own value in its output
 };
 
 constexpr int SCAN_CH = 8;          // tokens staged at a time
@@ -250,7 +240,8 @@ __device__ __forceinline__ float group_sum(float v) {
 
 // TA: type of a and k (the compute type for wkv's r and k, float for the delta rule's unit vectors); T: type of v.
 // FORGET: a holds silu(q) in float32, the decay is the forget gate f and the key is 1 - f (k and scalar are not used).
-// SSD: S_ij <- w_i S_ij + k_i v_j, then o_j = sum_i a_i S_ij + scalar v_j (the read sees the token's own write).
+// SSD: S_ij <- w S_ij + (dt k_i) v_j with one decay w for the head, then o_j = sum_i a_i S_ij + bonus_h v_j (the read sees
+// the token's own write); a and k are the convolved rows themselves (C and B of the head's group), of the compute type.
 template <typename TA, typename T, int NI16, int SPLIT, bool DELTA, bool FORGET = false, bool SSD = false>
 __global__ __launch_bounds__(WAVE) void scan_kernel(ScanArgs p) {
     constexpr int RP = NI16 * 4;                       // rows of the state's column a lane keeps
@@ -291,14 +282,16 @@ __global__ __launch_bounds__(WAVE) void scan_kernel(ScanArgs p) {
     // Addresses are a base that is the same for the whole wave (the chunk's first token, this head) plus a small
     // offset a lane: the rows of a chunk lie less than 2^31 elements apart.
     const int jc = min(j, Dv - 1);
-    const unsigned strideA = (unsigned)(Ha * D), strideW = (unsigned)(H * D), strideV = (unsigned)p.ldv, strideS = (unsigned)H;
+    const unsigned strideA = (unsigned)p.lda, strideW = (unsigned)(H * D), strideV = (unsigned)p.ldv, strideS = (unsigned)H;
+    const float bonus_h = SSD ? p.head_bonus[head] : 0.f;
+    float fd[CH];                                      // ssd: a token's decay
     int ic[PER];
 #pragma unroll
     for (int e = 0; e < PER; ++e) ic[e] = min(lane + e * WAVE, D - 1);
     auto fetch = [&](int first, int count) {
-        const TA* ba = pa + ((long long)first * Ha + ha) * D;
-        const TA* bk = pk + ((long long)first * Ha + ha) * D;
-        const float* bw = p.decay + ((long long)first * H + head) * D;
+        const TA* ba = pa + (long long)first * p.lda + (long long)ha * D;
+        const TA* bk = pk + (long long)first * p.lda + (long long)ha * D;
+        const float* bw = SSD ? p.decay + (long long)first * H + head : p.decay + ((long long)first * H + head) * D;
         const T* bv = pv + (long long)first * p.ldv + (long long)head * Dv;
         const float* bs = p.scalar + (long long)first * H + head;
 #pragma unroll
@@ -308,15 +301,16 @@ __global__ __launch_bounds__(WAVE) void scan_kernel(ScanArgs p) {
             for (int e = 0; e < PER; ++e) {
                 fa[tt][e] = ba[tc * strideA + (unsigned)ic[e]];
                 fk[tt][e] = bk[tc * strideA + (unsigned)ic[e]];
-                fw[tt][e] = bw[tc * strideW + (unsigned)ic[e]];
+                if (!SSD) fw[tt][e] = bw[tc * strideW + (unsigned)ic[e]];
             }
+            if (SSD) fd[tt] = bw[tc * strideS];
             fv[tt] = bv[tc * strideV + (unsigned)jc];
             fb[tt] = bs[tc * strideS];
         }
     };
     // one token: the state's rows of this lane move on and the token's output leaves.  Four partial sums a
     // lane (rows 0, 1, 2, 3 of every group of four), added in a fixed order, then the quad's exchange.
-    auto token = [&](int tt, float vt, float sc, float* orow) {
+    auto token = [&](int tt, float vt, float sc, float wt, float* orow) {
         float o4[4] = {0.f, 0.f, 0.f, 0.f};
         if (DELTA) {
             float kv4[4] = {0.f, 0.f, 0.f, 0.f};
@@ -344,12 +338,16 @@ __global__ __launch_bounds__(WAVE) void scan_kernel(ScanArgs p) {
         } else {
 #pragma unroll
             for (int g4 = 0; g4 < NI16; ++g4) {
-                const f32x4 w4 = *(const f32x4*)&sw[tt][row0 + g4 * 4];
+                const f32x4 zero4 = {0.f, 0.f, 0.f, 0.f};
+                const f32x4 w4 = SSD ? zero4 : *(const f32x4*)&sw[tt][row0 + g4 * 4];
                 const f32x4 k4 = *(const f32x4*)&sk[tt][row0 + g4 * 4];
                 const f32x4 r4 = *(const f32x4*)&sa[tt][row0 + g4 * 4];
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
-                    if (FORGET || SSD) {
+                    if (SSD) {
+                        s[g4 * 4 + e] = fmaf(wt, s[g4 * 4 + e], k4[e] * vt);
+                        o4[e] = fmaf(r4[e], s[g4 * 4 + e], o4[e]);
+                    } else if (FORGET) {
                         s[g4 * 4 + e] = fmaf(w4[e], s[g4 * 4 + e], k4[e] * vt);
                         o4[e] = fmaf(r4[e], s[g4 * 4 + e], o4[e]);
                     } else {
@@ -360,7 +358,8 @@ __global__ __launch_bounds__(WAVE) void scan_kernel(ScanArgs p) {
             }
         }
         float o = group_sum<SPLIT>((o4[0] + o4[1]) + (o4[2] + o4[3]));
-        if (!DELTA && !FORGET) o = fmaf(sc, vt, o);
+        if (SSD) o = fmaf(bonus_h, vt, o);
+        else if (!DELTA && !FORGET) o = fmaf(sc, vt, o);
         // (the lanes of a group hold the same sum and write it to the same place: no lane is switched off for it)
         if (jv) orow[(unsigned)tt * (unsigned)(H * Dv)] = o;
     };
@@ -368,19 +367,20 @@ __global__ __launch_bounds__(WAVE) void scan_kernel(ScanArgs p) {
     fetch(t0, min(n, CH));
     for (int c0 = 0; c0 < n; c0 += CH) {
         const int count = min(CH, n - c0);
-        float v[CH], sc[CH];
+        float v[CH], sc[CH], wd[CH];
 #pragma unroll
         for (int tt = 0; tt < CH; ++tt) {
             v[tt] = to_f32(fv[tt]);
             sc[tt] = fb[tt];
+            wd[tt] = SSD ? fd[tt] : 0.f;
 #pragma unroll
             for (int e = 0; e < PER; ++e) {
                 const int i = lane + e * WAVE;
                 const bool ok = i < D;                 // (tokens beyond the chunk's last are staged and never read)
                 if (i < DP) {
                     sa[tt][i] = ok ? to_f32(fa[tt][e]) : 0.f;
-                    sk[tt][i] = ok ? (FORGET ? 1.0f - fw[tt][e] : to_f32(fk[tt][e])) : 0.f;
-                    sw[tt][i] = ok ? fw[tt][e] : 0.f;
+                    sk[tt][i] = ok ? (FORGET ? 1.0f - fw[tt][e] : SSD ? fb[tt] * to_f32(fk[tt][e]) : to_f32(fk[tt][e])) : 0.f;
+                    if (!SSD) sw[tt][i] = ok ? fw[tt][e] : 0.f;
                 }
             }
         }
@@ -393,11 +393,11 @@ __global__ __launch_bounds__(WAVE) void scan_kernel(ScanArgs p) {
         float* orow = p.out + ((long long)(t0 + c0) * H + head) * Dv + j;     // this lane's place in the chunk's first row
         if (count == CH) {                             // eight whole tokens: no test between them
 #pragma unroll
-            for (int tt = 0; tt < CH; ++tt) token(tt, v[tt], sc[tt], orow);
+            for (int tt = 0; tt < CH; ++tt) token(tt, v[tt], sc[tt], wd[tt], orow);
         } else {
 #pragma unroll
             for (int tt = 0; tt < CH; ++tt)
-                if (tt < count) token(tt, v[tt], sc[tt], orow);
+                if (tt < count) token(tt, v[tt], sc[tt], wd[tt], orow);
         }
         __builtin_amdgcn_wave_barrier();               // the reads stay before the next tokens' writes
     }
@@ -509,7 +509,7 @@ TUFF_EXPORT int tuff_wkv_scan(const void* r, const void* k, const void* v, int d
     PrepArgs pp{r, k, lw, w0, u, nullptr, nullptr, 0, nullptr, nullptr, bonus, H, H, D, (long long)H * D};
     if (dt == DT_F32) hipLaunchKernelGGL((scan_prep_kernel<float, false>), dim3(n_tokens, H), dim3(WAVE), 0, stream, pp);
     else hipLaunchKernelGGL((scan_prep_kernel<bf16_t, false>), dim3(n_tokens, H), dim3(WAVE), 0, stream, pp);
-    ScanArgs p{r, k, v, lw, bonus, state, out, q_start, q_len, state_slot, H, H, D, D, (long long)H * D};
+    ScanArgs p{r, k, v, lw, bonus, state, out, q_start, q_len, state_slot, H, H, D, D, (long long)H * D, (long long)H * D, nullptr};
     return dt == DT_F32 ? launch_scan<float, float, false>(p, n_requests, stream)
                         : launch_scan<bf16_t, bf16_t, false>(p, n_requests, stream);
 }
@@ -530,7 +530,7 @@ TUFF_EXPORT int tuff_delta_scan(const void* q, const void* k, const void* v, int
     PrepArgs pp{q, k, a, dt_bias, A_log, b, a_head, ld_small, qn, kn, beta, H, Hk, D, ld};
     if (dt == DT_F32) hipLaunchKernelGGL((scan_prep_kernel<float, true>), dim3(n_tokens, H), dim3(WAVE), 0, stream, pp);
     else hipLaunchKernelGGL((scan_prep_kernel<bf16_t, true>), dim3(n_tokens, H), dim3(WAVE), 0, stream, pp);
-    ScanArgs p{qn, kn, v, a, beta, state, out, q_start, q_len, state_slot, H, H, D, Dv, ldv};
+    ScanArgs p{qn, kn, v, a, beta, state, out, q_start, q_len, state_slot, H, H, D, Dv, ldv, (long long)H * D, nullptr};
     return dt == DT_F32 ? launch_scan<float, float, true>(p, n_requests, stream)
                         : launch_scan<float, bf16_t, true>(p, n_requests, stream);
 }
@@ -552,22 +552,27 @@ TUFF_EXPORT int tuff_head_norm_gate(const float* o, const float* w, int w_stride
 
 // ssd (the state-space recurrence with a scalar decay per head): xbc holds a token's convolved rows
 // [x (H*P) | B (G*N) | C (G*N)] of type dt, ld elements apart; dt_raw float32, a token's H values ld_dt apart; dt_bias,
-// A_log, Dh float32 [H]; work arrays qn, kn, decay float32 [T][H*N] and bonus float32 [T][H]; state float32
-// [slots][H][N][P]; out float32 [T][H][P].  Head h reads group h / (H / G).
+// A_log, Dh float32 [H]; work arrays step and decay float32 [T][H]; state float32 [slots][H][N][P]; out float32
+// [T][H][P].  Head h reads B and C of group h / (H / G), from the rows as they lie.
 TUFF_EXPORT int tuff_ssd_scan(const void* xbc, int dt, long long ld, const float* dt_raw, long long ld_dt, const float* dt_bias,
-                              const float* A_log, const float* Dh, float* qn, float* kn, float* decay, float* bonus, float* state,
+                              const float* A_log, const float* Dh, float* step, float* decay, float* state,
                               float* out, const int* q_start, const int* q_len, const int* state_slot, int n_tokens, int n_requests,
                               int H, int G, int N, int P, hipStream_t stream) {
     if (n_requests <= 0 || n_tokens <= 0) return 0;
     if (H <= 0 || H > 65535 || G <= 0 || H % G || ld < (long long)H * P + 2LL * G * N || ld_dt < H) return -2;
-    const int b_off = H * P;
-    if (dt == DT_F32) hipLaunchKernelGGL(ssd_prep_kernel<float>, dim3(n_tokens, H), dim3(WAVE), 0, stream, (const float*)xbc, ld, b_off, dt_raw, ld_dt, dt_bias, A_log, Dh, qn, kn, decay, bonus, H, G, N);
-    else hipLaunchKernelGGL(ssd_prep_kernel<bf16_t>, dim3(n_tokens, H), dim3(WAVE), 0, stream, (const bf16_t*)xbc, ld, b_off, dt_raw, ld_dt, dt_bias, A_log, Dh, qn, kn, decay, bonus, H, G, N);
+    const long long n = (long long)n_tokens * H;
+    hipLaunchKernelGGL(ssd_prep_kernel, dim3((unsigned)ceil_div_ll(n, 256)), dim3(256), 0, stream, dt_raw, ld_dt, dt_bias, A_log, step, decay, n, H);
     int rc = launch_status();
     if (rc != 0) return rc;
-    ScanArgs p{qn, kn, xbc, decay, bonus, state, out, q_start, q_len, state_slot, H, H, N, P, ld};
-    return dt == DT_F32 ? launch_scan<float, float, false, false, true>(p, n_requests, stream)
-                        : launch_scan<float, bf16_t, false, false, true>(p, n_requests, stream);
+    const long long b_off = (long long)H * P, c_off = b_off + (long long)G * N;
+    if (dt == DT_F32) {
+        const float* x = (const float*)xbc;
+        ScanArgs p{x + c_off, x + b_off, x, decay, step, state, out, q_start, q_len, state_slot, H, G, N, P, ld, ld, Dh};
+        return launch_scan<float, float, false, false, true>(p, n_requests, stream);
+    }
+    const bf16_t* x = (const bf16_t*)xbc;
+    ScanArgs p{x + c_off, x + b_off, x, decay, step, state, out, q_start, q_len, state_slot, H, G, N, P, ld, ld, Dh};
+    return launch_scan<bf16_t, bf16_t, false, false, true>(p, n_requests, stream);
 }
 
 // forget: x rows [q (H*D) | z (H*D) | v (H*Dv)] of type dt, ld elements apart, as projected; bias (or null) and lower
@@ -585,7 +590,7 @@ TUFF_EXPORT int tuff_forget_scan(const void* x, int dt, long long ld, const floa
     if (rc != 0) return rc;
     // (k and the per-token scalar are loaded and not used: they point at arrays of the right reach)
     const void* v = dt == DT_F32 ? (const void*)((const float*)x + 2LL * HD) : (const void*)((const bf16_t*)x + 2LL * HD);
-    ScanArgs p{qn, qn, v, f, f, state, out, q_start, q_len, state_slot, H, H, D, Dv, ld};
+    ScanArgs p{qn, qn, v, f, f, state, out, q_start, q_len, state_slot, H, H, D, Dv, ld, (long long)H * D, nullptr};
     return dt == DT_F32 ? launch_scan<float, float, false, true>(p, n_requests, stream)
                         : launch_scan<float, bf16_t, false, true>(p, n_requests, stream);
 }

@@ -82,11 +82,11 @@ class LatentAttentionMixer(Mixer, PagedAttention):
 
     def weight_decls(self):
         n = self.names
-        decls = self.proj.weight_decls() + self.out.weight_decls() + [
-            WeightDecl(n["uk"], (self.H * self.dk, self.rank), "normal", role="projection"),
-            WeightDecl(n["uv"], (self.H * self.dv, self.rank), "normal", role="projection")]
+        decls = self.proj.weight_decls() + self.out.weight_decls()
         if self.own_rows:
             decls.append(WeightDecl(n["dkv.norm"], (self.rank,), "norm"))
+        decls += [WeightDecl(n["uk"], (self.H * self.dk, self.rank), "normal", role="projection"),
+                  WeightDecl(n["uv"], (self.H * self.dv, self.rank), "normal", role="projection")]
         if self.has_sink:
             decls.append(WeightDecl(n["sink"], (self.H,), "normal"))
         return decls
