@@ -270,12 +270,17 @@ def test_configuration_reads_every_size_and_refuses_what_it_cannot_run():
         lambda r: r["layers"][1]["mlp"]["router"].update(top=9),
         lambda r: r["layers"][1]["mlp"]["router"]["groups"].update(count=3),
         lambda r: r["layers"][1]["mlp"]["router"]["groups"].update(keep=1),          # four chosen of the two experts kept
-        lambda r: r["layers"][1]["mlp"]["router"].pop("scale"),
+        lambda r: r["layers"][1]["mlp"]["router"].update(scale="large"),
         lambda r: r["layers"][0]["mlp"].update(kind="gated"),
         lambda r: r["norm"].update(eps=0),
         lambda r: r.update(logit_softcap=-1.0),
         lambda r: r.pop("vocab"),
     ]
+    # a router without groups or scale: one group of all experts, plain scores
+    bare = copy.deepcopy(xu.X_MIXED)
+    bare["layers"][3]["mlp"]["router"] = {"experts": 4, "top": 2}
+    ffn = build_model(config_from_dict(bare)).blocks[3].ffn
+    assert (ffn.route_groups, ffn.route_keep, ffn.route_scale) == (1, 1, 1.0)
     for i, spoil in enumerate(bad):
         raw = copy.deepcopy(xu.X_MIXED)
         spoil(raw)

@@ -12,6 +12,7 @@ config.json is nested:
         type "latent_attention":  mixer {heads, dim, vdim, kv_rank, scale, kv_from (optional: the layer whose latent rows it reads)}
         mlp {kind: "dense", ff}
         mlp {kind: "moe", router: {experts, top, scale, groups: {count, keep}}, expert: {ff}}
+            (without router.groups the choice is not limited; without router.scale the weights are the plain scores)
 """
 from __future__ import annotations
 
@@ -104,8 +105,9 @@ class KinelixConfig(ModelConfig):
             return
         try:
             r = mlp["router"]
-            sizes = [r["experts"], r["top"], mlp["expert"]["ff"], r["groups"]["count"], r["groups"]["keep"]]
-            scale = r["scale"]
+            groups = r.setdefault("groups", {"count": 1, "keep": 1})       # no groups named: one group of all experts, kept
+            sizes = [r["experts"], r["top"], mlp["expert"]["ff"], groups["count"], groups["keep"]]
+            scale = r.setdefault("scale", 1.0)
         except (KeyError, TypeError) as e:
             raise ConfigError(f"{where}.mlp lacks a key ({e})") from None
         if not all(_is_int(v) for v in sizes):

@@ -144,6 +144,7 @@ __global__ __launch_bounds__(PN_THREADS) void scale_add_layer_norm_kernel(
     constexpr int N = EPT > 0 ? EPT : 1;
     float xv[N];
     float sum = 0.f;
+    float nv[N];                                       // the next norm's weight: asked for with everything else, before the first sum
     if (EPT > 0) {
         float yv[N], lv[N];
 #pragma unroll
@@ -153,6 +154,7 @@ __global__ __launch_bounds__(PN_THREADS) void scale_add_layer_norm_kernel(
             xv[k] = in ? x[src + c] : 0.f;
             yv[k] = (in && y) ? y[src + c] : 0.f;
             lv[k] = (in && y) ? ls[c] : 0.f;
+            nv[k] = (in && h_out) ? w_next[c] : 0.f;
         }
 #pragma unroll
         for (int k = 0; k < N; ++k) {
@@ -193,7 +195,7 @@ __global__ __launch_bounds__(PN_THREADS) void scale_add_layer_norm_kernel(
 #pragma unroll
         for (int k = 0; k < N; ++k) {
             const int c = threadIdx.x + k * PN_THREADS;
-            if (c < d) h_out[dst + c] = from_f32<T>((xv[k] - mean) * inv * w_next[c]);
+            if (c < d) h_out[dst + c] = from_f32<T>((xv[k] - mean) * inv * nv[k]);
         }
     } else {
         for (int c = threadIdx.x; c < d; c += PN_THREADS) h_out[dst + c] = from_f32<T>((x[src + c] - mean) * inv * w_next[c]);
