@@ -81,6 +81,8 @@ ONLY = {
     "mamba": config(48, 101, [layer(mamba(4, 8, 16, 2, 2, 4))], embed_scale=3.0),
     "mamba_one_tap": config(48, 101, [layer(mamba(2, 20, 12, 2, 1, 1))]),
     "mamba_wide_state": config(64, 101, [layer(mamba(2, 8, 72, 1, 2, 3))]),         # sixteen lanes a value channel
+    # sizes the chunked form takes (multiples of 16): prompt portions of 64 tokens and more run on the matrix cores
+    "mamba_sixteens": config(64, 101, [layer(mamba(4, 16, 32, 2, 1, 4)), layer(mamba(2, 48, 48, 1, 2, 2))], embed_scale=2.0),
     "delta": config(48, 101, [layer(delta(4, 2, 16, 8, 3))]),
     "delta_wide": config(64, 101, [layer(delta(2, 2, 80, 72, 2))]),
     "latent": config(48, 101, [layer(latent(2, 16, 24, 32, 0.6))]),

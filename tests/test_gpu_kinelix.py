@@ -238,7 +238,7 @@ def test_peaky_attention_far_keys_in_prompts_and_in_decoding(gpu, dtype):
 def test_states_that_remember_hundreds_of_tokens(gpu, dtype):
     """The recurrent mixers alone over long prompts cut at odd places and decoded: some heads decay by a hundredth a
     token, so a state that was lost, cleared or taken from a neighbour's slot shows hundreds of tokens later."""
-    for name in ("only_mamba", "only_delta", "only_mamba_wide_state"):
+    for name in ("only_mamba", "only_delta", "only_mamba_wide_state", "only_mamba_sixteens"):
         reqs = requests(name, [400, 260], seed=9)
         check(name, dtype, util.plan_tail(reqs, tail=40), reqs)
         check(name, dtype, util.plan_chunks(reqs, sizes=(3, 1, 2, 64, 5, 129, 8, 7, 2)), reqs)
@@ -387,6 +387,60 @@ def test_state_space_scan_alone_across_cuts(gpu, H, G, N, P):
         for r in (0, 1):
             assert (got[r].double() - want[r]).abs().max() < 2e-4 * max(1.0, float(want[r].abs().max())), (cuts, r)
         assert torch.isnan(state[0]).all() and torch.isnan(state[2]).all() and torch.isnan(state[4]).all()
+
+
+@pytest.mark.parametrize("H, G, N, P", [(4, 2, 16, 16), (2, 1, 48, 48), (6, 3, 128, 64), (3, 1, 32, 64)])
+def test_state_space_recurrence_in_chunks_against_token_by_token(gpu, H, G, N, P):
+    """The chunked form on the matrix cores (bfloat16 rows, steps with prompt portions) against the float64 recurrence and
+    the token-by-token kernel: requests of 1 to 300 tokens side by side, chunks that are full, partial and of one token,
+    states that start at zero and not, slots between slots of NaN; then a second step that goes on from the first's states."""
+    from tuff_amd.csrc import ops
+    assert ops.ssd_chunked_supported(torch.bfloat16, N, P)
+    g = torch.Generator().manual_seed(H * N + P)
+    lens_all = [300, 1, 64, 65, 7, 129]
+    C = H * P + 2 * G * N
+    dt_bias, A_log, D = torch.randn(H, generator=g), torch.randn(H, generator=g) * 1.5 - 2.0, torch.randn(H, generator=g)
+    rows = [(torch.randn(n, C + 8, generator=g) * 0.7).to(torch.bfloat16) for n in lens_all]
+    dts = [torch.randn(n, H + 3, generator=g) for n in lens_all]
+
+    def exact(r, S0):
+        n = lens_all[r]
+        x = rows[r][:, :H * P].double().view(n, H, P)
+        B = rows[r][:, H * P:H * P + G * N].double().view(n, G, N)
+        Cm = rows[r][:, H * P + G * N:C].double().view(n, G, N)
+        dt = plain.softplus(dts[r][:, 1:1 + H].double() + dt_bias.double())
+        dec = torch.exp(-torch.exp(A_log.double()) * dt)
+        y = torch.zeros(n, H, P, dtype=torch.float64)
+        S = S0.clone()
+        for h in range(H):
+            for t in range(n):
+                S[h] = dec[t, h] * S[h] + dt[t, h] * torch.outer(B[t, h // (H // G)], x[t, h])
+                y[t, h] = S[h].T @ Cm[t, h // (H // G)] + D[h].double() * x[t, h]
+        return y.reshape(n, H * P), S
+    R = len(lens_all)
+    slots = [2 * r + 1 for r in range(R)]
+    state = torch.full((2 * R + 1, H, N, P), float("nan"), device=gpu)
+    start = [torch.randn(H, N, P, generator=g) * (r % 2) for r in range(R)]          # every second request starts from zero
+    for r in range(R):
+        state[slots[r]] = start[r].to(gpu)
+    serial = state.clone()
+    step, _ = _step_tensors(gpu, lens_all, slots)
+    x_all, dt_all = torch.cat(rows).to(gpu), torch.cat(dts).to(gpu)
+    S_now = [s_.double() for s_ in start]
+    for round_ in range(2):                                # the second step goes on from the states the first left
+        out, out_serial = torch.zeros(sum(lens_all), H * P, device=gpu), torch.zeros(sum(lens_all), H * P, device=gpu)
+        args = (x_all[:, :C], dt_all[:, 1:1 + H], dt_bias.to(gpu), A_log.to(gpu), D.to(gpu))
+        ops.ssd_chunked(*args, state, out, H=H, G=G, N=N, P=P, **step)
+        ops.ssd_scan(*args, serial, out_serial, H=H, G=G, N=N, P=P, **step)
+        at = 0
+        for r, n in enumerate(lens_all):
+            want, S_now[r] = exact(r, S_now[r])
+            scale = max(1.0, float(want.abs().max()))
+            assert (out[at:at + n].double().cpu() - want).abs().max() < 3e-4 * scale, (round_, r)
+            assert (out_serial[at:at + n].double().cpu() - want).abs().max() < 3e-4 * scale, (round_, r)
+            assert (state[slots[r]].double().cpu() - S_now[r]).abs().max() < 3e-4 * max(1.0, float(S_now[r].abs().max())), (round_, r)
+            at += n
+        assert all(torch.isnan(state[2 * r]).all() for r in range(R + 1))
 
 
 @pytest.mark.parametrize("H, Hk, D, Dv", [(4, 2, 16, 8), (3, 1, 10, 6), (2, 2, 80, 72)])

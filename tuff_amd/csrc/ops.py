@@ -57,6 +57,9 @@ _SIGNATURES = {
         "tuff_ssd_scan": [_c_void_p, _c_int, _c_ll, _c_void_p, _c_ll, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p,
                           _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int,
                           _c_int, _c_void_p],
+        "tuff_ssd_chunked": [_c_void_p, _c_ll, _c_void_p, _c_ll, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p,
+                             _c_void_p, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int,
+                             _c_int, _c_int, _c_void_p],
         "tuff_forget_scan": [_c_void_p, _c_int, _c_ll, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p,
                              _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p],
     },
@@ -1643,6 +1646,42 @@ def ssd_scan(xbc, dt_raw, dt_bias, A_log, D_skip, state, out, *, q_start, q_len,
         _gpu("state", state, torch.float32, (None, H, N, P)), _gpu("out", out, torch.float32, (T, H * P)),
         _gpu("q_start", q_start, torch.int32, (R,)), _gpu("q_len", q_len, torch.int32, (R,)),
         _gpu("state_slot", state_slot, torch.int32, (R,)), T, R, H, G, N, P, _stream()), "ssd_scan")
+
+
+SSD_CHUNK = 64                   # tokens a chunk of ssd_chunked
+
+
+def ssd_chunked_supported(dtype, N: int, P: int) -> bool:
+    """Whether the chunked form takes these sizes: bfloat16 rows, state and head sizes that are multiples of 16, a state of
+    at most 128 and heads of at most 64 channels (what a workgroup's 64 KB of LDS hold)."""
+    return dtype == torch.bfloat16 and N % 16 == 0 and P % 16 == 0 and 0 < N <= 128 and 0 < P <= 64
+
+
+def ssd_chunked(xbc, dt_raw, dt_bias, A_log, D_skip, state, out, *, q_start, q_len, state_slot, H, G, N, P) -> None:
+    """ssd_scan's recurrence for prompt portions in chunks of 64 tokens on the matrix cores (float32 matrix instructions;
+    all factors, sums and the state float32): the same function, its sums in another order.  xbc bfloat16; the other
+    arguments as for ssd_scan."""
+    T = xbc.shape[0]
+    R = q_start.shape[0]
+    if not ssd_chunked_supported(xbc.dtype, N, P):
+        raise KernelError(f"ssd_chunked: bfloat16 rows, a state of {N} (a multiple of 16 up to 128) and heads of {P} (up to 64) channels")
+    if G < 1 or H % G:
+        raise KernelError(f"ssd_chunked: {H} heads in {G} groups")
+    ld = _rows_view("xbc", xbc, H * P + 2 * G * N)
+    ld_dt = _rows_view("dt_raw", dt_raw, H)
+    if dt_raw.dtype != torch.float32:
+        raise KernelError("ssd_chunked: dt_raw must be float32")
+    chunks = -(-T // SSD_CHUNK) + R
+    small = torch.empty(3 * T * H + chunks * H, dtype=torch.float32, device=xbc.device)      # step sizes, decays, their logarithms; chunk decays
+    U = torch.empty(chunks, H, N, P, dtype=torch.float32, device=xbc.device)
+    at = lambda i: small.data_ptr() + 4 * i * T * H
+    _check(load("recurrent").tuff_ssd_chunked(
+        xbc.data_ptr(), ld, dt_raw.data_ptr(), ld_dt, _gpu("dt_bias", dt_bias, torch.float32, (H,)),
+        _gpu("A_log", A_log, torch.float32, (H,)), _gpu("D_skip", D_skip, torch.float32, (H,)),
+        at(0), at(1), at(2), U.data_ptr(), at(3), chunks,
+        _gpu("state", state, torch.float32, (None, H, N, P)), _gpu("out", out, torch.float32, (T, H * P)),
+        _gpu("q_start", q_start, torch.int32, (R,)), _gpu("q_len", q_len, torch.int32, (R,)),
+        _gpu("state_slot", state_slot, torch.int32, (R,)), T, R, H, G, N, P, _stream()), "ssd_chunked")
 
 
 def forget_scan(x, bias, lower, state, out, *, q_start, q_len, state_slot, H, D, Dv) -> None:

@@ -195,15 +195,249 @@ __global__ void forget_prep_kernel(const T* __restrict__ x, long long ld, const 
 // What enters the state-space recurrence besides the convolved rows, float32 [T][H] each: the step size
 // dt = softplus(dt_raw + dt_bias_h) and the decay exp(-exp(A_log_h) dt), one number for all state channels of a head.
 // dt_raw float32, a token's H values ld_dt apart.
+// log_decay (or null): the decay's logarithm, -exp(A_log_h) dt, for the chunked form.
 __global__ void ssd_prep_kernel(const float* __restrict__ dt_raw, long long ld_dt, const float* __restrict__ dt_bias,
-                                const float* __restrict__ A_log, float* __restrict__ dt_out, float* __restrict__ decay, long long n, int H) {
+                                const float* __restrict__ A_log, float* __restrict__ dt_out, float* __restrict__ decay,
+                                float* __restrict__ log_decay, long long n, int H) {
     const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= n) return;
     const long long t = i / H;
     const int head = (int)(i % H);
     const float dt = softplusf_(dt_raw[t * ld_dt + head] + dt_bias[head]);
+    const float la = -expf(A_log[head]) * dt;
     dt_out[i] = dt;
-    decay[i] = expf(-expf(A_log[head]) * dt);
+    decay[i] = expf(la);
+    if (log_decay) log_decay[i] = la;
+}
+
+// ------------------------------------------------- the state-space recurrence in chunks, on the matrix cores
+// For prompt portions in bfloat16 runs.  A request's tokens of the step are cut into chunks of 64 from the portion's
+// first token.  With a_t the running sum of the decays' logarithms inside a chunk (a_t <= 0, falling), K_s = dt_s B_s and
+// S_in the state at the chunk's start:
+//     y_t = sum_{s <= t} exp(a_t - a_s) (C_t . K_s) x_s  +  exp(a_t) C_t^T S_in  +  D x_t
+//     S_out = exp(a_last) S_in + sum_s exp(a_last - a_s) K_s x_s^T
+// Three kernels: (1) every chunk's own contribution U = sum_s exp(a_last - a_s) K_s x_s^T and its decay exp(a_last), all
+// chunks at once; (2) per request and head the chunks in order, an element of the state a thread: S_in of every chunk
+// takes U's place, the last S_out goes to the slot; (3) every chunk's outputs, all chunks at once.  All factors, sums and
+// the state are float32; the products run as float32 matrix instructions (16 x 16 x 4), whose operands are the float32
+// values themselves (B, C and x are bfloat16 as the convolution left them, converted exactly).  Every exponent is <= 0.
+// The sums of a token are formed in another order than token by token, so a position's result depends on where its
+// portion began, within float32 rounding; a float32 run keeps the token-by-token kernel.
+constexpr int CHUNK = 64;
+
+__device__ __forceinline__ f32x4 mfma_f32(float a, float b, f32x4 c) { return __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, c, 0, 0, 0); }
+
+struct SsdChunkArgs {
+    const bf16_t* xbc;              // a token's rows [x (H*P) | B (G*N) | C (G*N)], ld apart
+    long long ld;
+    const float *dt, *la;           // [T][H]: step size, logarithm of the decay
+    const float* Dh;                // [H]
+    float* state;                   // [slots][H][N][P]
+    float* U;                       // [chunks][H][N][P]: a chunk's contribution, then the state at its start
+    float* cdec;                    // [chunks][H]: exp(a_last)
+    float* out;                     // [T][H][P]
+    const int *q_start, *q_len, *state_slot;
+    int R, H, G, N, P;
+};
+
+// Which request and which of its chunks workgroup `ci` takes (chunks are numbered request after request); false: none.
+__device__ __forceinline__ bool chunk_of(const SsdChunkArgs& p, int ci, int& r, int& t0, int& L) {
+    for (r = 0; r < p.R; ++r) {
+        const int n = p.q_len[r];
+        const int nc = (n + CHUNK - 1) / CHUNK;
+        if (ci < nc) {
+            t0 = p.q_start[r] + ci * CHUNK;
+            L = min(CHUNK, n - ci * CHUNK);
+            return true;
+        }
+        ci -= nc;
+    }
+    return false;
+}
+
+// a[t] = sum_{s <= t} la[s] over the chunk's tokens, by the first wave; sa[CHUNK] in LDS (a[t] = a[L-1] beyond the chunk)
+__device__ __forceinline__ void chunk_prefix(const SsdChunkArgs& p, int t0, int L, int head, float* sa) {
+    if (threadIdx.x < WAVE) {
+        const int lane = threadIdx.x;
+        float v = lane < L ? p.la[(long long)(t0 + lane) * p.H + head] : 0.f;
+#pragma unroll
+        for (int off = 1; off < WAVE; off *= 2) {
+            const float up = __shfl_up(v, off, WAVE);
+            if (lane >= off) v += up;
+        }
+        sa[lane] = v;
+    }
+}
+
+// A lane's operands of consecutive matrix instructions lie side by side in LDS: the inner index of a product may be
+// taken in any order as long as both operands agree, so lane group q (of four) takes the q-th quarter of it, and its
+// operands of four instructions are one 16-byte (float32) or 8-byte (bfloat16) read.
+__global__ __launch_bounds__(256) void ssd_chunk_state_kernel(SsdChunkArgs p) {
+    extern __shared__ __attribute__((aligned(16))) float sm[];
+    const int N = p.N, P = p.P, head = blockIdx.y, tid = threadIdx.x;
+    int r, t0, L;
+    if (!chunk_of(p, blockIdx.x, r, t0, L)) return;
+    constexpr int LDS_ = CHUNK + 4;
+    float* sa = sm;                               // [CHUNK]
+    float* sw = sa + CHUNK;                       // [CHUNK]: exp(a_last - a_s) dt_s
+    float* sBt = sw + CHUNK;                      // [N][CHUNK + 4]: w_s B_s[n], a state channel's tokens side by side
+    float* sXt = sBt + N * LDS_;                  // [P][CHUNK + 4]
+    chunk_prefix(p, t0, L, head, sa);
+    __syncthreads();
+    if (tid < CHUNK) sw[tid] = tid < L ? expf(sa[L - 1] - sa[tid]) * p.dt[(long long)(t0 + tid) * p.H + head] : 0.f;
+    __syncthreads();
+    const int g = head / (p.H / p.G);
+    const bf16_t* base = p.xbc + (long long)t0 * p.ld;
+    const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+    const int NC = N / 8, PC = P / 8;
+    for (int i = tid; i < CHUNK * NC; i += 256) {
+        const int s_ = i / NC, ch = i % NC;
+        const bf16x8 v = s_ < L ? *(const bf16x8*)(base + (long long)s_ * p.ld + (long long)p.H * P + (long long)g * N + ch * 8) : zero8;
+        const float w = sw[s_];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) sBt[(ch * 8 + e) * LDS_ + s_] = w * (float)v[e];
+    }
+    for (int i = tid; i < CHUNK * PC; i += 256) {
+        const int s_ = i / PC, ch = i % PC;
+        const bf16x8 v = s_ < L ? *(const bf16x8*)(base + (long long)s_ * p.ld + (long long)head * P + ch * 8) : zero8;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) sXt[(ch * 8 + e) * LDS_ + s_] = (float)v[e];
+    }
+    __syncthreads();
+    const int wave = tid / WAVE, lane = tid % WAVE, l16 = lane % 16, lq = lane / 16;
+    const int NT = N / 16, PT = P / 16;
+    float* U = p.U + ((long long)blockIdx.x * p.H + head) * N * P;
+    for (int tile = wave; tile < NT * PT; tile += 4) {
+        const int nt = tile / PT, pt = tile % PT;
+        f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+        const float* pa = sBt + (nt * 16 + l16) * LDS_ + lq * (CHUNK / 4);
+        const float* pb = sXt + (pt * 16 + l16) * LDS_ + lq * (CHUNK / 4);
+#pragma unroll
+        for (int j4 = 0; j4 < CHUNK / 16; ++j4) {
+            const f32x4 a4 = *(const f32x4*)(pa + 4 * j4), b4 = *(const f32x4*)(pb + 4 * j4);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) acc = mfma_f32(a4[e], b4[e], acc);
+        }
+#pragma unroll
+        for (int e = 0; e < 4; ++e) U[(long long)(nt * 16 + 4 * lq + e) * P + pt * 16 + l16] = acc[e];
+    }
+    if (tid == 0) p.cdec[(long long)blockIdx.x * p.H + head] = expf(sa[L - 1]);
+}
+
+__global__ __launch_bounds__(256) void ssd_state_pass_kernel(SsdChunkArgs p) {
+    const int r = blockIdx.x, head = blockIdx.y;
+    const int n = p.q_len[r];
+    if (n <= 0) return;
+    const long long NP = (long long)p.N * p.P;
+    const long long e = (long long)blockIdx.z * 256 + threadIdx.x;
+    if (e >= NP) return;
+    int first = 0;
+    for (int r2 = 0; r2 < r; ++r2) first += (p.q_len[r2] + CHUNK - 1) / CHUNK;
+    const int nc = (n + CHUNK - 1) / CHUNK;
+    float* S = p.state + ((long long)p.state_slot[r] * p.H + head) * NP + e;
+    float s_ = *S;
+    for (int c = 0; c < nc; ++c) {
+        float* u = p.U + ((long long)(first + c) * p.H + head) * NP + e;
+        const float own = *u;
+        *u = s_;
+        s_ = fmaf(p.cdec[(long long)(first + c) * p.H + head], s_, own);
+    }
+    *S = s_;
+}
+
+__global__ __launch_bounds__(256) void ssd_chunk_out_kernel(SsdChunkArgs p) {
+    extern __shared__ __attribute__((aligned(16))) float sm[];
+    const int N = p.N, P = p.P, head = blockIdx.y, tid = threadIdx.x;
+    int r, t0, L;
+    if (!chunk_of(p, blockIdx.x, r, t0, L)) return;
+    constexpr int LDG = CHUNK + 4, LDXT = CHUNK + 8;
+    const int ldn = N + 8;
+    float* sa = sm;                               // [CHUNK]
+    float* sdt = sa + CHUNK;                      // [CHUNK]
+    float* sGt = sdt + CHUNK;                     // [CHUNK (t)][CHUNK + 4 (s)]: the masked, scaled C_t . B_s
+    bf16_t* sB = (bf16_t*)(sGt + CHUNK * LDG);    // [CHUNK][N + 8]
+    bf16_t* sC = sB + CHUNK * ldn;                // [CHUNK][N + 8]
+    bf16_t* sXt = sC + CHUNK * ldn;               // [P][CHUNK + 8]: a channel's tokens side by side
+    chunk_prefix(p, t0, L, head, sa);
+    if (tid >= 64 && tid < 128) sdt[tid - 64] = tid - 64 < L ? p.dt[(long long)(t0 + tid - 64) * p.H + head] : 0.f;
+    const int g = head / (p.H / p.G);
+    const bf16_t* base = p.xbc + (long long)t0 * p.ld;
+    const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+    const int NC = N / 8, PC = P / 8;
+    for (int i = tid; i < CHUNK * NC; i += 256) {
+        const int s_ = i / NC, ch = i % NC;
+        const bf16_t* row = base + (long long)s_ * p.ld + (long long)p.H * P + (long long)g * N + ch * 8;
+        *(bf16x8*)(sB + s_ * ldn + ch * 8) = s_ < L ? *(const bf16x8*)row : zero8;
+        *(bf16x8*)(sC + s_ * ldn + ch * 8) = s_ < L ? *(const bf16x8*)(row + (long long)p.G * N) : zero8;
+    }
+    for (int i = tid; i < CHUNK * PC; i += 256) {
+        const int s_ = i / PC, ch = i % PC;
+        const bf16x8 v = s_ < L ? *(const bf16x8*)(base + (long long)s_ * p.ld + (long long)head * P + ch * 8) : zero8;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) sXt[(ch * 8 + e) * LDXT + s_] = v[e];
+    }
+    __syncthreads();
+    const int wave = tid / WAVE, lane = tid % WAVE, l16 = lane % 16, lq = lane / 16;
+    const int nq = N / 4;                          // a lane group's share of the state channels
+    // Gt[t][s] = (s <= t) exp(a_t - a_s) dt_s sum_n B[s][n] C[t][n]; tiles above the diagonal are zero
+    for (int tile = wave; tile < 16; tile += 4) {
+        const int st = tile / 4, tt = tile % 4;
+        f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+        if (st <= tt && st * 16 < L) {
+            const bf16_t* pa = sB + (st * 16 + l16) * ldn + lq * nq;
+            const bf16_t* pb = sC + (tt * 16 + l16) * ldn + lq * nq;
+#pragma unroll 4
+            for (int j4 = 0; j4 < nq / 4; ++j4) {
+                const bf16x4 a4 = *(const bf16x4*)(pa + 4 * j4), b4 = *(const bf16x4*)(pb + 4 * j4);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) acc = mfma_f32((float)a4[e], (float)b4[e], acc);
+            }
+        }
+        const int t = tt * 16 + l16;
+        f32x4 gv;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const int s_ = st * 16 + 4 * lq + e;
+            gv[e] = (s_ <= t && t < L) ? acc[e] * expf(sa[t] - sa[s_]) * sdt[s_] : 0.f;
+        }
+        *(f32x4*)(sGt + t * LDG + st * 16 + 4 * lq) = gv;
+    }
+    __syncthreads();
+    // y[t][c] = sum_s Gt[t][s] x[s][c] + exp(a_t) sum_n C[t][n] S_in[n][c] + D x[t][c]
+    const float* Sin = p.U + ((long long)blockIdx.x * p.H + head) * N * P;
+    const float dh = p.Dh[head];
+    const int PT = P / 16;
+    for (int tile = wave; tile < 4 * PT; tile += 4) {
+        const int tt = tile / PT, pt = tile % PT;
+        if (tt * 16 >= L) continue;
+        f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+        const int sq = 4 * (tt + 1);               // a lane group's share of the keys up to the tile's last row
+        const float* pg = sGt + (tt * 16 + l16) * LDG + lq * sq;
+        const bf16_t* px = sXt + (pt * 16 + l16) * LDXT + lq * sq;
+        for (int j4 = 0; j4 <= tt; ++j4) {
+            const f32x4 a4 = *(const f32x4*)(pg + 4 * j4);
+            const bf16x4 b4 = *(const bf16x4*)(px + 4 * j4);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) acc = mfma_f32(a4[e], (float)b4[e], acc);
+        }
+        const float ea = expf(sa[min(tt * 16 + l16, L - 1)]);
+        const bf16_t* pc = sC + (tt * 16 + l16) * ldn + lq * nq;
+        const float* ps = Sin + (long long)(lq * nq) * P + pt * 16 + l16;
+#pragma unroll 2
+        for (int j4 = 0; j4 < nq / 4; ++j4) {
+            const bf16x4 c4 = *(const bf16x4*)(pc + 4 * j4);
+            float s4[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) s4[e] = ps[(long long)(4 * j4 + e) * P];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) acc = mfma_f32(ea * (float)c4[e], s4[e], acc);
+        }
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const int t = tt * 16 + 4 * lq + e, c = pt * 16 + l16;
+            if (t < L) p.out[((long long)(t0 + t) * p.H + head) * P + c] = fmaf(dh, (float)sXt[c * LDXT + t], acc[e]);
+        }
+    }
 }
 
 struct ScanArgs {
@@ -561,7 +795,7 @@ TUFF_EXPORT int tuff_ssd_scan(const void* xbc, int dt, long long ld, const float
     if (n_requests <= 0 || n_tokens <= 0) return 0;
     if (H <= 0 || H > 65535 || G <= 0 || H % G || ld < (long long)H * P + 2LL * G * N || ld_dt < H) return -2;
     const long long n = (long long)n_tokens * H;
-    hipLaunchKernelGGL(ssd_prep_kernel, dim3((unsigned)ceil_div_ll(n, 256)), dim3(256), 0, stream, dt_raw, ld_dt, dt_bias, A_log, step, decay, n, H);
+    hipLaunchKernelGGL(ssd_prep_kernel, dim3((unsigned)ceil_div_ll(n, 256)), dim3(256), 0, stream, dt_raw, ld_dt, dt_bias, A_log, step, decay, (float*)nullptr, n, H);
     int rc = launch_status();
     if (rc != 0) return rc;
     const long long b_off = (long long)H * P, c_off = b_off + (long long)G * N;
@@ -573,6 +807,31 @@ TUFF_EXPORT int tuff_ssd_scan(const void* xbc, int dt, long long ld, const float
     const bf16_t* x = (const bf16_t*)xbc;
     ScanArgs p{x + c_off, x + b_off, x, decay, step, state, out, q_start, q_len, state_slot, H, G, N, P, ld, ld, Dh};
     return launch_scan<bf16_t, bf16_t, false, false, true>(p, n_requests, stream);
+}
+
+// The same recurrence in chunks of 64 tokens on the matrix cores (see above), for bfloat16 rows: N and P multiples of 16,
+// N <= 128, P <= 64.  Work arrays: step, decay, log_decay float32 [T][H]; U float32 [chunks][H][N][P] and cdec float32
+// [chunks][H] with chunks >= ceil(T / 64) + requests (what the step's portions can be cut into at most).
+TUFF_EXPORT int tuff_ssd_chunked(const void* xbc, long long ld, const float* dt_raw, long long ld_dt, const float* dt_bias,
+                                 const float* A_log, const float* Dh, float* step, float* decay, float* log_decay, float* U, float* cdec,
+                                 int chunks, float* state, float* out, const int* q_start, const int* q_len, const int* state_slot,
+                                 int n_tokens, int n_requests, int H, int G, int N, int P, hipStream_t stream) {
+    if (n_requests <= 0 || n_tokens <= 0) return 0;
+    if (H <= 0 || H > 65535 || G <= 0 || H % G || ld < (long long)H * P + 2LL * G * N || ld_dt < H) return -2;
+    if (N % 16 || P % 16 || N > 128 || P > 64 || N <= 0 || P <= 0 || chunks < ceil_div(n_tokens, CHUNK) + n_requests || n_requests > 65535) return -2;
+    const long long n = (long long)n_tokens * H;
+    hipLaunchKernelGGL(ssd_prep_kernel, dim3((unsigned)ceil_div_ll(n, 256)), dim3(256), 0, stream, dt_raw, ld_dt, dt_bias, A_log, step, decay, log_decay, n, H);
+    int rc = launch_status();
+    if (rc != 0) return rc;
+    SsdChunkArgs p{(const bf16_t*)xbc, ld, step, log_decay, Dh, state, U, cdec, out, q_start, q_len, state_slot, n_requests, H, G, N, P};
+    if (ld % 8 || ((unsigned long long)xbc & 15)) return -2;         // the rows are read 16 bytes at a time
+    const size_t lds1 = (size_t)(2 * CHUNK + (N + P) * (CHUNK + 4)) * sizeof(float);
+    const size_t lds3 = (size_t)(2 * CHUNK + CHUNK * (CHUNK + 4)) * sizeof(float) + (size_t)(2 * CHUNK * (N + 8) + P * (CHUNK + 8)) * sizeof(bf16_t);
+    if (lds1 > 65536 || lds3 > 65536) return -2;
+    hipLaunchKernelGGL(ssd_chunk_state_kernel, dim3(chunks, H), dim3(256), lds1, stream, p);
+    hipLaunchKernelGGL(ssd_state_pass_kernel, dim3(n_requests, H, (unsigned)ceil_div_ll((long long)N * P, 256)), dim3(256), 0, stream, p);
+    hipLaunchKernelGGL(ssd_chunk_out_kernel, dim3(chunks, H), dim3(256), lds3, stream, p);
+    return launch_status();
 }
 
 // forget: x rows [q (H*D) | z (H*D) | v (H*Dv)] of type dt, ld elements apart, as projected; bias (or null) and lower

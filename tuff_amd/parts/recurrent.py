@@ -332,8 +332,11 @@ class Mamba2Mixer(Mixer):
         ops.conv_act(raw, self.taps, None if tail is None else tail.state, xbc, req_of_token=ctx.req_of_token,
                      q_len=ctx.q_len, activation="silu", bias=self.conv_b, **step)
         o = torch.empty(T, self.inner, dtype=torch.float32, device=h.device)
-        ops.ssd_scan(xbc, dt, self.dt_bias, self.A_log, self.D_skip, S.state, o, q_len=ctx.q_len, H=self.H, G=self.G,
-                     N=self.N, P=self.P, **step)
+        # a step with prompt portions (of 64 tokens and more in all): the recurrence in chunks on the matrix cores, where
+        # its sizes fit; single tokens, short steps and float32 runs: token by token
+        chunked = ctx.max_q_len > 1 and T >= ops.SSD_CHUNK and ops.ssd_chunked_supported(xbc.dtype, self.N, self.P)
+        (ops.ssd_chunked if chunked else ops.ssd_scan)(xbc, dt, self.dt_bias, self.A_log, self.D_skip, S.state, o, q_len=ctx.q_len,
+                                                       H=self.H, G=self.G, N=self.N, P=self.P, **step)
         y = self.rt.empty(T, self.inner)
         ops.head_norm_gate(o, self.norm_w, z, y, H=self.norm_groups, Dv=self.inner // self.norm_groups, eps=self.eps,
                            per_head_weight=True, gate_activation="silu", gate_first=True)
