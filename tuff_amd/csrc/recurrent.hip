@@ -407,35 +407,40 @@ __global__ __launch_bounds__(256) void ssd_chunk_out_kernel(SsdChunkArgs p) {
     const float* Sin = p.U + ((long long)blockIdx.x * p.H + head) * N * P;
     const float dh = p.Dh[head];
     const int PT = P / 16;
-    for (int tile = wave; tile < 4 * PT; tile += 4) {
-        const int tt = tile / PT, pt = tile % PT;
-        if (tt * 16 >= L) continue;
-        f32x4 acc = {0.f, 0.f, 0.f, 0.f};
-        const int sq = 4 * (tt + 1);               // a lane group's share of the keys up to the tile's last row
-        const float* pg = sGt + (tt * 16 + l16) * LDG + lq * sq;
-        const bf16_t* px = sXt + (pt * 16 + l16) * LDXT + lq * sq;
-        for (int j4 = 0; j4 <= tt; ++j4) {
-            const f32x4 a4 = *(const f32x4*)(pg + 4 * j4);
-            const bf16x4 b4 = *(const bf16x4*)(px + 4 * j4);
-#pragma unroll
-            for (int e = 0; e < 4; ++e) acc = mfma_f32(a4[e], (float)b4[e], acc);
-        }
-        const float ea = expf(sa[min(tt * 16 + l16, L - 1)]);
-        const bf16_t* pc = sC + (tt * 16 + l16) * ldn + lq * nq;
+    // a wave takes a block of 16 channels and walks the chunk's four blocks of tokens with it: its share of S_in's
+    // columns (a lane group's quarter of the state channels, at most 32 numbers a lane) is read once, into registers
+    for (int pt = wave; pt < PT; pt += 4) {
         const float* ps = Sin + (long long)(lq * nq) * P + pt * 16 + l16;
-#pragma unroll 2
-        for (int j4 = 0; j4 < nq / 4; ++j4) {
-            const bf16x4 c4 = *(const bf16x4*)(pc + 4 * j4);
-            float s4[4];
+        float sreg[32];
 #pragma unroll
-            for (int e = 0; e < 4; ++e) s4[e] = ps[(long long)(4 * j4 + e) * P];
+        for (int k = 0; k < 32; ++k) sreg[k] = k < nq ? ps[(long long)k * P] : 0.f;
+        const bf16_t* px = sXt + (pt * 16 + l16) * LDXT;
+        for (int tt = 0; tt < 4; ++tt) {
+            if (tt * 16 >= L) break;
+            f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+            const int sq = 4 * (tt + 1);           // a lane group's share of the keys up to the block's last row
+            const float* pg = sGt + (tt * 16 + l16) * LDG + lq * sq;
+            for (int j4 = 0; j4 <= tt; ++j4) {
+                const f32x4 a4 = *(const f32x4*)(pg + 4 * j4);
+                const bf16x4 b4 = *(const bf16x4*)(px + lq * sq + 4 * j4);
 #pragma unroll
-            for (int e = 0; e < 4; ++e) acc = mfma_f32(ea * (float)c4[e], s4[e], acc);
-        }
+                for (int e = 0; e < 4; ++e) acc = mfma_f32(a4[e], (float)b4[e], acc);
+            }
+            const float ea = expf(sa[min(tt * 16 + l16, L - 1)]);
+            const bf16_t* pc = sC + (tt * 16 + l16) * ldn + lq * nq;
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
-            const int t = tt * 16 + 4 * lq + e, c = pt * 16 + l16;
-            if (t < L) p.out[((long long)(t0 + t) * p.H + head) * P + c] = fmaf(dh, (float)sXt[c * LDXT + t], acc[e]);
+            for (int j4 = 0; j4 < 8; ++j4) {
+                if (4 * j4 < nq) {
+                    const bf16x4 c4 = *(const bf16x4*)(pc + 4 * j4);
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) acc = mfma_f32(ea * (float)c4[e], sreg[4 * j4 + e], acc);
+                }
+            }
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const int t = tt * 16 + 4 * lq + e, c = pt * 16 + l16;
+                if (t < L) p.out[((long long)(t0 + t) * p.H + head) * P + c] = fmaf(dh, (float)sXt[c * LDXT + t], acc[e]);
+            }
         }
     }
 }
