@@ -76,7 +76,6 @@ X_PLAIN = config(48, 101, [
     layer(delta(2, 1, 24, 24, 3), moe(4, 2, 24, 2, 2, 1.2)),
     layer(latent(2, 8, 8, 16, 0.35), moe(4, 2, 24, 2, 1, 1.0)),
 ], softcap=1.0)
-_L = layer(latent(1, 8, 8, 8, 0.3))
 ONLY = {
     "mamba": config(48, 101, [layer(mamba(4, 8, 16, 2, 2, 4))], embed_scale=3.0),
     "mamba_one_tap": config(48, 101, [layer(mamba(2, 20, 12, 2, 1, 1))]),
