@@ -217,10 +217,16 @@ def test_long_decoding(gpu, dtype):
     assert eng.graph_replays > 0                           # steps of single tokens were recorded and replayed
 
 
-def test_steps_of_portions_recorded_in_sections(gpu):
-    reqs = requests("mixed", [96, 96, 96, 96], seed=7)
-    plan = util.plan_chunks(reqs, sizes=(8,))
-    eng, _ = check("mixed", "float32", plan, reqs)
+@pytest.mark.parametrize("name, dtype, size", [("mixed", "float32", 8), ("only_mamba_sixteens", "bfloat16", 32),
+                                               ("only_latent_shared", "float32", 16)])
+def test_steps_of_portions_recorded_in_sections(gpu, name, dtype, size):
+    """Steps of one size that keep coming are recorded in sections and replayed; with portions of 32 tokens of four
+    requests the state-space recurrence runs in chunks inside the recorded sections (its grids are sized by the step's
+    tokens and slots alone)."""
+    reqs = requests(name, [192, 192, 192, 192], seed=7)
+    plan = [{"step": k, "entries": [{"id": rid, "tokens": toks[k * size:(k + 1) * size], "want": list(range(size))} for rid, toks in reqs.items()],
+             "end": list(reqs) if (k + 1) * size == 192 else []} for k in range(192 // size)]        # the four side by side
+    eng, _ = check(name, dtype, plan, reqs)
     assert eng.section_replays > 0
 
 
