@@ -228,7 +228,7 @@ __global__ __launch_bounds__(DEC_KEYS) void decode_scores_kernel(
     int H, int Hkv, int hd, int page_size, int window, float scale, const float* __restrict__ slopes,
     const float* __restrict__ log_r1, const float* __restrict__ log_r2, int n_parts, int chunks) {
     __shared__ float qs[DEC_HEADS * 256];
-    __shared__ float scratch[4];
+    __shared__ float red_m[DEC_HEADS * 4], red_l[DEC_HEADS * 4];      // the four waves' maxima and sums of every head
     // (a group of more than GC heads is shared out among `chunks` workgroups, GC heads at a time each)
     const int t = blockIdx.x, kvh = blockIdx.y / chunks, chunk = blockIdx.y % chunks, part = blockIdx.z, tid = threadIdx.x;
     const int G = H / Hkv;
@@ -284,24 +284,44 @@ __global__ __launch_bounds__(DEC_KEYS) void decode_scores_kernel(
                 }
             }
         }
+        // The part's maximum and sum of every head: the waves' own maxima (sums) of all heads first, then one exchange
+        // through LDS for all of them, where a reduction a head at a time would cross the workgroup's barrier twice a
+        // head.  The waves' values meet in the order of block_max_256 and block_sum_256: the same bits.
+        float sv[GC], red[GC];
 #pragma unroll
         for (int g = 0; g < GC; ++g) {
-            if (g >= Gc) break;                                 // uniform
-            const int head = head0 + g;
+            const int head = head0 + min(g, Gc - 1);
             float s = -INFINITY;
-            if (valid) {
+            if (valid && g < Gc) {
                 s = acc[g] * scale;
                 if (slopes) s -= slopes[head] * dist;
                 if (log_r1) s -= log_r1[head] * log1pf(log_r2[head] * dist);
                 S[((long long)t * H + head) * n_parts * DEC_KEYS + key] = s;
             }
-            const float m = block_max_256(s, scratch);
-            const float l = block_sum_256(valid ? expf(s - m) : 0.f, scratch);
-            if (tid == 0) {
-                float* dst = ml + (((long long)t * H + head) * n_parts + part) * 2;
-                dst[0] = m;
-                dst[1] = l;
-            }
+            sv[g] = s;
+            red[g] = wave_max(s);
+        }
+        __syncthreads();                                        // (everybody has read qs; red_m and red_l are free)
+        if (tid % WAVE == 0) {
+#pragma unroll
+            for (int g = 0; g < GC; ++g) red_m[g * 4 + tid / WAVE] = red[g];
+        }
+        __syncthreads();
+        float m[GC];
+#pragma unroll
+        for (int g = 0; g < GC; ++g) {
+            m[g] = fmaxf(fmaxf(red_m[g * 4], red_m[g * 4 + 1]), fmaxf(red_m[g * 4 + 2], red_m[g * 4 + 3]));
+            red[g] = wave_sum((valid && g < Gc) ? expf(sv[g] - m[g]) : 0.f);
+        }
+        if (tid % WAVE == 0) {
+#pragma unroll
+            for (int g = 0; g < GC; ++g) red_l[g * 4 + tid / WAVE] = red[g];
+        }
+        __syncthreads();
+        if (tid < Gc) {
+            float* dst = ml + (((long long)t * H + head0 + tid) * n_parts + part) * 2;
+            dst[0] = fmaxf(fmaxf(red_m[tid * 4], red_m[tid * 4 + 1]), fmaxf(red_m[tid * 4 + 2], red_m[tid * 4 + 3]));
+            dst[1] = (red_l[tid * 4] + red_l[tid * 4 + 1]) + (red_l[tid * 4 + 2] + red_l[tid * 4 + 3]);
         }
     }
 }
